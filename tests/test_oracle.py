@@ -1,0 +1,172 @@
+"""Pins the CPU oracle (numpy, C, torch port) without the reference code:
+brute-force loops on tiny shapes, closed-form special cases, adjointness, linearity,
+autograd through an independent forward, finite differences and the fp8 decode table."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import egs_oracle as O
+from oracle import c_oracle as C
+from oracle import torch_port as P
+
+
+def rand_case(seed, B, T, E, K, I, J, replace=True):
+    g = np.random.default_rng(seed)
+    X = g.standard_normal((B, T, I))
+    Wg = g.standard_normal((E, I, J)) / np.sqrt(I)
+    Ws = g.standard_normal((E, J, I)) / np.sqrt(J)
+    if replace:
+        Ind = g.integers(0, T, size=(B, E, K))
+    else:
+        Ind = np.stack([np.stack([g.permutation(T)[:K] for _ in range(E)]) for _ in range(B)])
+    Y = g.standard_normal((B, E, K, J))
+    dOut = g.standard_normal((B, T, I))
+    return X, Wg, Ws, Ind.astype(np.int64), Y, dOut
+
+
+TINY = [(1, 1, 1, 1, 1, 1), (2, 3, 2, 4, 3, 2), (3, 4, 3, 2, 4, 3), (2, 5, 1, 7, 2, 5), (1, 2, 4, 3, 5, 1)]
+
+
+@pytest.mark.parametrize("shape", TINY)
+def test_vectorised_matches_brute_force(shape):
+    X, Wg, Ws, Ind, Y, dOut = rand_case(7, *shape)
+    T = shape[1]
+    np.testing.assert_allclose(O.gather_forward(X, Wg, Ind), O.brute_gather_forward(X, Wg, Ind), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(O.scatter_forward(Y, Ws, Ind, T), O.brute_scatter_forward(Y, Ws, Ind, T), rtol=1e-12, atol=1e-12)
+    dX, dW = O.gather_backward(X, Wg, Ind, Y)
+    bX, bW = O.brute_gather_backward(X, Wg, Ind, Y)
+    np.testing.assert_allclose(dX, bX, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dW, bW, rtol=1e-12, atol=1e-12)
+    dY, dWs = O.scatter_backward(Y, Ws, Ind, dOut)
+    bY, bWs = O.brute_scatter_backward(Y, Ws, Ind, dOut)
+    np.testing.assert_allclose(dY, bY, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(dWs, bWs, rtol=1e-12, atol=1e-12)
+
+
+def test_hand_computed_known_answer():
+    # one batch, two tokens, one expert picking token 1 twice and token 0 once
+    X = np.array([[[1.0, 2.0], [3.0, 4.0]]])                 # [1,2,2]
+    W = np.array([[[1.0, 0.0, 2.0], [0.0, 1.0, -1.0]]])      # [1,2,3]
+    Ind = np.array([[[1, 1, 0]]])
+    Y = O.gather_forward(X, W, Ind)
+    expect = np.array([[[[3.0, 4.0, 2.0], [3.0, 4.0, 2.0], [1.0, 2.0, 0.0]]]])
+    np.testing.assert_array_equal(Y, expect)
+    Ws = np.array([[[1.0, 1.0], [0.0, 2.0], [1.0, 0.0]]])    # [1,3,2]
+    out = O.scatter_forward(Y, Ws, Ind, 2)
+    # row picks: [3,4,2]@Ws = [5, 11]; twice into token 1; [1,2,0]@Ws=[1,5] into token 0
+    np.testing.assert_array_equal(out, np.array([[[1.0, 5.0], [10.0, 22.0]]]))
+
+
+def test_identity_routing_reduces_to_matmul():
+    g = np.random.default_rng(3)
+    B, T, I, J = 3, 9, 5, 4
+    X = g.standard_normal((B, T, I)); W = g.standard_normal((1, I, J))
+    Ind = np.broadcast_to(np.arange(T)[None, None, :], (B, 1, T)).copy()
+    np.testing.assert_allclose(O.gather_forward(X, W, Ind)[:, 0], X @ W[0], rtol=1e-13, atol=1e-13)
+    Y = g.standard_normal((B, 1, T, J)); Ws = g.standard_normal((1, J, I))
+    np.testing.assert_allclose(O.scatter_forward(Y, Ws, Ind, T), Y[:, 0] @ Ws[0], rtol=1e-13, atol=1e-13)
+
+
+def test_scatter_of_gather_counts_picks():
+    # W_g @ W_s = identity and every token picked c(t) times => out = c(t) * X
+    g = np.random.default_rng(5)
+    B, T, E, K, I = 2, 6, 3, 4, 5
+    X = g.standard_normal((B, T, I))
+    Q = np.linalg.qr(g.standard_normal((I, I)))[0]
+    Wg = np.broadcast_to(Q, (E, I, I)).copy(); Ws = np.broadcast_to(Q.T, (E, I, I)).copy()
+    Ind = g.integers(0, T, size=(B, E, K))
+    out = O.scatter_forward(O.gather_forward(X, Wg, Ind), Ws, Ind, T)
+    cnt = np.zeros((B, T))
+    for b in range(B):
+        np.add.at(cnt[b], Ind[b].ravel(), 1)
+    np.testing.assert_allclose(out, cnt[..., None] * X, rtol=1e-12, atol=1e-12)
+    assert (out[cnt == 0] == 0).all()
+
+
+def test_adjointness_and_linearity():
+    X, Wg, Ws, Ind, Y, dOut = rand_case(11, 3, 7, 4, 5, 6, 3)
+    T = 7
+    G = Y
+    lhs = (O.gather_forward(X, Wg, Ind) * G).sum()
+    rhs = (X * O.scatter_forward(G, np.swapaxes(Wg, 1, 2), Ind, T)).sum()
+    assert abs(lhs - rhs) <= 1e-10 * abs(lhs)
+    X2 = rand_case(12, 3, 7, 4, 5, 6, 3)[0]
+    np.testing.assert_allclose(O.gather_forward(2 * X - 3 * X2, Wg, Ind),
+                               2 * O.gather_forward(X, Wg, Ind) - 3 * O.gather_forward(X2, Wg, Ind), atol=1e-12)
+    # permuting k inside (b,e) leaves the scatter output unchanged
+    perm = np.random.default_rng(1).permutation(5)
+    np.testing.assert_allclose(O.scatter_forward(Y[:, :, perm], Ws, Ind[:, :, perm], T),
+                               O.scatter_forward(Y, Ws, Ind, T), atol=1e-12)
+
+
+@pytest.mark.parametrize("shape", [(2, 5, 3, 4, 6, 3), (3, 17, 5, 9, 13, 7), (4, 33, 2, 40, 8, 19)])
+def test_c_restatement_matches_numpy(shape):
+    X, Wg, Ws, Ind, Y, dOut = rand_case(21, *shape)
+    T = shape[1]
+    f = lambda a: a.astype(np.float32)
+    X, Wg, Ws, Y, dOut = map(f, (X, Wg, Ws, Y, dOut))
+    np.testing.assert_allclose(C.gather(X, Wg, Ind), O.gather_forward(X, Wg, Ind), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(C.scatter(Y, Ws, Ind, T), O.scatter_forward(Y, Ws, Ind, T), rtol=1e-12, atol=1e-12)
+    dX, dW = O.gather_backward(X, Wg, Ind, Y)
+    np.testing.assert_allclose(C.scatter(Y, Wg, Ind, T, C.W_EIJ), dX, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(C.dw(X, Y, Ind, C.W_EIJ), dW, rtol=1e-12, atol=1e-12)
+    dY, dWs = O.scatter_backward(Y, Ws, Ind, dOut)
+    np.testing.assert_allclose(C.gather(dOut, Ws, Ind, C.W_EJI), dY, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(C.dw(dOut, Y, Ind, C.W_EJI), dWs, rtol=1e-12, atol=1e-12)
+    with pytest.raises(IndexError):
+        bad = Ind.copy(); bad[0, 0, 0] = T
+        C.gather(X, Wg, bad)
+
+
+def test_torch_port_and_autograd_match_closed_forms():
+    X, Wg, Ws, Ind, Y, dOut = rand_case(31, 3, 11, 4, 6, 7, 5)
+    T = 11
+    t = lambda a: torch.from_numpy(a)
+    np.testing.assert_allclose(P.gather(t(X), t(Wg), t(Ind)).numpy(), O.gather_forward(X, Wg, Ind), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(P.scatter(t(Y), t(Ws), t(Ind), T).numpy(), O.scatter_forward(Y, Ws, Ind, T), rtol=1e-12, atol=1e-12)
+    # autograd through the torch forward vs the oracle's closed-form backward
+    Xt = t(X).requires_grad_(True); Wt = t(Wg).requires_grad_(True)
+    P.gather(Xt, Wt, t(Ind)).backward(t(Y))
+    dX, dW = O.gather_backward(X, Wg, Ind, Y)
+    np.testing.assert_allclose(Xt.grad.numpy(), dX, rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(Wt.grad.numpy(), dW, rtol=1e-11, atol=1e-11)
+    Yt = t(Y).requires_grad_(True); Wst = t(Ws).requires_grad_(True)
+    P.scatter(Yt, Wst, t(Ind), T).backward(t(dOut))
+    dY, dWs = O.scatter_backward(Y, Ws, Ind, dOut)
+    np.testing.assert_allclose(Yt.grad.numpy(), dY, rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(Wst.grad.numpy(), dWs, rtol=1e-11, atol=1e-11)
+    # whole chain
+    Yc, outc, dXc, dWgc, dWsc = P.chain_fwd_bwd(t(X), t(Wg), t(Ws), t(Ind), t(dOut))
+    Yo = O.gather_forward(X, Wg, Ind); outo = O.scatter_forward(Yo, Ws, Ind, T)
+    dYo, dWso = O.scatter_backward(Yo, Ws, Ind, dOut); dXo, dWgo = O.gather_backward(X, Wg, Ind, dYo)
+    for a, b in ((Yc, Yo), (outc, outo), (dXc, dXo), (dWgc, dWgo), (dWsc, dWso)):
+        np.testing.assert_allclose(a.numpy(), b, rtol=1e-10, atol=1e-10)
+
+
+def test_finite_difference_of_loss():
+    X, Wg, Ws, Ind, Y, dOut = rand_case(41, 2, 5, 3, 4, 3, 2)
+    G = Y
+    loss = lambda X_, W_: (O.gather_forward(X_, W_, Ind) * G).sum()
+    dX, dW = O.gather_backward(X, Wg, Ind, G)
+    eps = 1e-6
+    for idx in [(0, 1, 2), (1, 4, 0)]:
+        Xp = X.copy(); Xp[idx] += eps; Xm = X.copy(); Xm[idx] -= eps
+        assert abs((loss(Xp, Wg) - loss(Xm, Wg)) / (2 * eps) - dX[idx]) < 1e-6
+    for idx in [(0, 0, 1), (2, 2, 0)]:
+        Wp = Wg.copy(); Wp[idx] += eps; Wm = Wg.copy(); Wm[idx] -= eps
+        assert abs((loss(X, Wp) - loss(X, Wm)) / (2 * eps) - dW[idx]) < 1e-6
+
+
+def test_fp8_decode_table_matches_torch():
+    bits = np.arange(256, dtype=np.uint8)
+    ours = O.fp8_e4m3fn_to_float(bits)
+    theirs = torch.from_numpy(bits).view(torch.float8_e4m3fn).to(torch.float32).numpy().astype(np.float64)
+    nan = np.isnan(theirs)
+    assert (np.isnan(ours) == nan).all()
+    np.testing.assert_array_equal(ours[~nan], theirs[~nan])
+    assert ours[0x7E] == 448.0 and ours[0x08] == 2.0 ** -6 and ours[0x01] == 2.0 ** -9
+
+
+def test_bf16_rounding_matches_torch():
+    a = np.random.default_rng(0).standard_normal(4096).astype(np.float32) * 37
+    np.testing.assert_array_equal(O.round_to_bf16(a), torch.from_numpy(a).to(torch.bfloat16).to(torch.float32).numpy())
