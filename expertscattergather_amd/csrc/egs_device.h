@@ -1,0 +1,214 @@
+// Device-side building blocks shared by the gfx950 kernels: 16-byte chunk loads with
+// tail/alignment guards, the swizzled K-major LDS tile, in-register block transposes,
+// MFMA steps per element type and index decoding.
+//
+// Vocabulary used throughout:
+//   pick    one (b, e, k) entry of Ind; picks of one expert form the rows m = b*K + k of a
+//           dense per-expert matrix product
+//   chunk   16 bytes = VEC consecutive elements along the reduction axis
+//   slab    BK reduction elements staged in LDS at a time
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace egs {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kThreads = 256;   // 4 wavefronts of 64 lanes per workgroup
+constexpr int kWave = 64;
+
+// ---------------------------------------------------------------------------- element types
+struct ElemF32 {
+    static constexpr int ES = 4;      // bytes per element
+    static constexpr int VEC = 4;     // elements per 16-byte chunk
+    static constexpr int ID = 0;
+};
+struct ElemF16 {
+    static constexpr int ES = 2;
+    static constexpr int VEC = 8;
+    static constexpr int ID = 1;
+};
+struct ElemBF16 {
+    static constexpr int ES = 2;
+    static constexpr int VEC = 8;
+    static constexpr int ID = 2;
+};
+
+__device__ __forceinline__ uint32_t f32_bits(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float bits_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// round-to-nearest-even float -> bf16 bits
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f)
+{
+    uint32_t u = f32_bits(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;      // NaN
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f)
+{
+    _Float16 h = (_Float16)f;
+    return (uint32_t)__builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return bits_f32(h << 16); }
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
+{
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+}
+
+template <class TT> __device__ __forceinline__ uint32_t f32_to_elem_bits(float f);
+template <> __device__ __forceinline__ uint32_t f32_to_elem_bits<ElemF32>(float f) { return f32_bits(f); }
+template <> __device__ __forceinline__ uint32_t f32_to_elem_bits<ElemF16>(float f) { return f32_to_f16_bits(f); }
+template <> __device__ __forceinline__ uint32_t f32_to_elem_bits<ElemBF16>(float f) { return f32_to_bf16_bits(f); }
+
+// one MFMA "chunk step": every lane supplies one 16-byte chunk per operand; lane group
+// g = lane/16 supplies reduction elements [g*VEC, g*VEC+VEC) of a 4*VEC wide step, rows /
+// columns are lane%16.  The accumulator holds rows 4*g..4*g+3 of column lane%16, where
+// "rows" index the first operand's lanes and "columns" the second operand's.
+template <class TT> __device__ __forceinline__ void mma_chunk(f32x4 &acc, const u32x4 &p, const u32x4 &q);
+template <> __device__ __forceinline__ void mma_chunk<ElemBF16>(f32x4 &acc, const u32x4 &p, const u32x4 &q)
+{
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, p), __builtin_bit_cast(bf16x8, q), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma_chunk<ElemF16>(f32x4 &acc, const u32x4 &p, const u32x4 &q)
+{
+    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, p), __builtin_bit_cast(f16x8, q), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void mma_chunk<ElemF32>(f32x4 &acc, const u32x4 &p, const u32x4 &q)
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(bits_f32(p[c]), bits_f32(q[c]), acc, 0, 0, 0);
+}
+
+// ---------------------------------------------------------------------------- index decode
+// Ind is read in its own integer width and never narrowed; returns -1 for out-of-range.
+__device__ __forceinline__ int64_t load_index_raw(const void *ind, int ind_dtype, int64_t at)
+{
+    switch (ind_dtype) {
+    case 0: return (int64_t) reinterpret_cast<const int16_t *>(ind)[at];
+    case 1: return (int64_t) reinterpret_cast<const int32_t *>(ind)[at];
+    case 2: return reinterpret_cast<const int64_t *>(ind)[at];
+    default: return (int64_t) reinterpret_cast<const uint8_t *>(ind)[at];
+    }
+}
+__device__ __forceinline__ int32_t load_token(const void *ind, int ind_dtype, int64_t at, int32_t T)
+{
+    int64_t t = load_index_raw(ind, ind_dtype, at);
+    return (t < 0 || t >= (int64_t)T) ? -1 : (int32_t)t;
+}
+
+// ---------------------------------------------------------------------------- guarded chunk loads
+// `row` points at element 0 of a source row (nullptr => the row reads as zeros), `k0` is the
+// first element wanted and `klim` the number of valid elements in the row.  `vec_ok` says the
+// row start is 16-byte aligned and k0 is a multiple of VEC, so an in-range chunk is one load.
+template <int ES>
+__device__ __forceinline__ u32x4 load_chunk(const char *row, int k0, int klim, bool vec_ok)
+{
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row == nullptr || k0 >= klim) return v;
+    constexpr int VEC = 16 / ES;
+    if (vec_ok && k0 + VEC <= klim) {
+        return *reinterpret_cast<const u32x4 *>(row + (size_t)k0 * ES);
+    }
+    if constexpr (ES == 2) {
+        const uint16_t *p = reinterpret_cast<const uint16_t *>(row) + k0;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            uint32_t h = (k0 + x < klim) ? (uint32_t)p[x] : 0u;
+            v[x >> 1] |= h << (16 * (x & 1));
+        }
+    } else {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(row) + k0;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = (k0 + x < klim) ? p[x] : 0u;
+    }
+    return v;
+}
+
+// 8 consecutive fp8 (OCP e4m3fn) bytes -> 8 bf16 in one chunk.  Exact: e4m3 has 3 mantissa bits.
+__device__ __forceinline__ u32x4 fp8x8_to_bf16_chunk(uint32_t lo, uint32_t hi)
+{
+    u32x4 v;
+    auto a = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, false);
+    auto b = __builtin_amdgcn_cvt_pk_f32_fp8((int)lo, true);
+    auto c = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, false);
+    auto d = __builtin_amdgcn_cvt_pk_f32_fp8((int)hi, true);
+    v[0] = (f32_bits(a[0]) >> 16) | (f32_bits(a[1]) & 0xffff0000u);
+    v[1] = (f32_bits(b[0]) >> 16) | (f32_bits(b[1]) & 0xffff0000u);
+    v[2] = (f32_bits(c[0]) >> 16) | (f32_bits(c[1]) & 0xffff0000u);
+    v[3] = (f32_bits(d[0]) >> 16) | (f32_bits(d[1]) & 0xffff0000u);
+    return v;
+}
+// fp8 source row, result is a bf16 chunk (8 elements); same guards as load_chunk.
+__device__ __forceinline__ u32x4 load_chunk_fp8_as_bf16(const char *row, int k0, int klim, bool vec_ok)
+{
+    u32x4 z = {0u, 0u, 0u, 0u};
+    if (row == nullptr || k0 >= klim) return z;
+    uint32_t lo = 0, hi = 0;
+    if (vec_ok && k0 + 8 <= klim) {
+        u32x2 w = *reinterpret_cast<const u32x2 *>(row + k0);
+        lo = w[0]; hi = w[1];
+    } else {
+        const uint8_t *p = reinterpret_cast<const uint8_t *>(row) + k0;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            uint32_t b = (k0 + x < klim) ? (uint32_t)p[x] : 0u;
+            if (x < 4) lo |= b << (8 * x); else hi |= b << (8 * (x - 4));
+        }
+    }
+    return fp8x8_to_bf16_chunk(lo, hi);
+}
+
+// ---------------------------------------------------------------------------- LDS tile
+// A tile holds ROWS rows of BK reduction elements, K-major (a row's chunks are adjacent), so
+// an MFMA operand fragment is one 16-byte LDS read per lane.  Chunk positions inside each
+// 128-byte group are XOR-swizzled by the row so that both the row-wise staging writes, the
+// transposed staging writes (8 rows apart) and the fragment reads (consecutive rows) spread
+// over the banks.
+template <int CH>   // chunks per row, power of two
+__device__ __forceinline__ int tile_chunk_index(int row, int c)
+{
+    constexpr int SW = (CH >= 8 ? 8 : CH) - 1;
+    return row * CH + (c ^ ((row ^ (row >> 3)) & SW));
+}
+
+// VEC x VEC block transpose in registers: in[r] holds VEC consecutive n of source row r;
+// out[c] holds the VEC consecutive r of column c.
+__device__ __forceinline__ void transpose8x8_16b(const u32x4 (&in)[8], u32x4 (&out)[8])
+{
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            uint32_t lo = in[2 * p][c >> 1], hi = in[2 * p + 1][c >> 1];
+            out[c][p] = (c & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+        }
+    }
+}
+__device__ __forceinline__ void transpose4x4_32b(const u32x4 (&in)[4], u32x4 (&out)[4])
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) out[c][r] = in[r][c];
+}
+
+// workgroup id -> (expert, tile): consecutive workgroup ids land on consecutive XCDs (8 per
+// device), so expert = 8*group + (id % 8) keeps all tiles of one expert on one XCD and its
+// weight tile in that XCD's L2.
+__device__ __forceinline__ bool decode_expert_tile(int bid, int tiles_per_expert, int E, int &e, int &tile)
+{
+    int xcd = bid & 7, slot = bid >> 3;
+    int eg = slot / tiles_per_expert;
+    tile = slot - eg * tiles_per_expert;
+    e = eg * 8 + xcd;
+    return e < E;
+}
+
+}  // namespace egs

@@ -1,0 +1,515 @@
+// Host side of the C ABI declared in include/egs_hip.h: argument validation, launch
+// planning (tile shapes, batch split of the weight gradient, workspace layout) and the
+// kernel launches.  No torch types, no device allocation, no synchronisation.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/egs_hip.h"
+#include "egs_device.h"
+#include "egs_rows_gemm.h"
+#include "egs_dw.h"
+#include "egs_scatter_aux.h"
+
+using namespace egs;
+
+namespace {
+
+thread_local char g_hip_error[256] = "";
+
+int hip_fail(hipError_t err, const char *what)
+{
+    snprintf(g_hip_error, sizeof(g_hip_error), "%s: %s", what, hipGetErrorString(err));
+    return EGS_ERR_HIP;
+}
+
+#define EGS_CHECK_LAUNCH(what)                                         \
+    do {                                                               \
+        hipError_t err__ = hipGetLastError();                          \
+        if (err__ != hipSuccess) return hip_fail(err__, what);         \
+    } while (0)
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+int elem_size(int dtype)
+{
+    switch (dtype) {
+    case EGS_F32: return 4;
+    case EGS_F16: case EGS_BF16: return 2;
+    case EGS_FP8_E4M3: return 1;
+    default: return 0;
+    }
+}
+bool act_dtype_ok(int d) { return d == EGS_F32 || d == EGS_F16 || d == EGS_BF16; }
+bool ind_dtype_ok(int d) { return d >= EGS_IND_I16 && d <= EGS_IND_U8; }
+bool layout_ok(int l) { return l == EGS_W_EIJ || l == EGS_W_EJI; }
+bool mode_ok(int m) { return m == EGS_SCATTER_DETERMINISTIC || m == EGS_SCATTER_ATOMIC; }
+
+int check_dims(const egs_dims *d)
+{
+    if (d == nullptr) return EGS_ERR_NULL_POINTER;
+    if (d->B < 0 || d->T < 0 || d->E < 0 || d->K < 0 || d->I < 0 || d->J < 0) return EGS_ERR_BAD_SHAPE;
+    // row counts and per-batch pick counts are held in 32-bit ints inside the kernels
+    if ((int64_t)d->B * d->K > INT32_MAX || (int64_t)d->E * d->K > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+    if ((int64_t)d->B * d->T > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+    return EGS_OK;
+}
+
+int grid_1d(size_t items, int cap = 8192)
+{
+    size_t g = (items + kThreads - 1) / kThreads;
+    if (g < 1) g = 1;
+    return (int)(g > (size_t)cap ? (size_t)cap : g);
+}
+
+// ------------------------------------------------------------------------------ plans
+struct ScatterPlan {
+    size_t seg_off_at, perm_at, cnt_at, rows_at;   // byte offsets inside the workspace
+    size_t bytes;
+};
+
+ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
+{
+    ScatterPlan pl = {0, 0, 0, 0, 0};
+    const size_t N = (size_t)d->E * d->K;
+    if (mode == EGS_SCATTER_ATOMIC) {
+        pl.rows_at = 0;
+        pl.bytes = act_dtype == EGS_F32 ? 0 : align_up((size_t)d->B * d->T * d->I * 4, 256);
+        return pl;
+    }
+    size_t at = 0;
+    pl.seg_off_at = at; at += align_up((size_t)d->B * ((size_t)d->T + 1) * 4, 256);
+    pl.perm_at = at;    at += align_up((size_t)d->B * N * 4, 256);
+    pl.cnt_at = at;     at += d->T > kCsrLdsTokens ? align_up((size_t)d->B * d->T * 4, 256) : 0;
+    pl.rows_at = at;    at += align_up((size_t)d->B * N * d->I * 4, 256);
+    pl.bytes = at;
+    return pl;
+}
+
+struct DwPlan {
+    int BI, BJ, BK, i_tiles, j_tiles, S, rows_per_split;
+    size_t bytes;
+};
+
+DwPlan plan_dw(const egs_dims *d, int act_dtype)
+{
+    DwPlan pl;
+    pl.BI = 128; pl.BJ = 64;
+    pl.BK = act_dtype == EGS_F32 ? 32 : 64;
+    pl.i_tiles = ceil_div(d->I, pl.BI);
+    pl.j_tiles = ceil_div(d->J, pl.BJ);
+    const int64_t Me = (int64_t)d->B * d->K;
+    const int64_t base = (int64_t)d->E * pl.i_tiles * pl.j_tiles;
+    int64_t S = base > 0 ? (512 + base - 1) / base : 1;
+    const int64_t max_s = Me > 0 ? (Me + pl.BK - 1) / pl.BK : 1;
+    if (S > max_s) S = max_s;
+    if (S > 64) S = 64;
+    if (S < 1) S = 1;
+    int64_t rows = Me > 0 ? (Me + S - 1) / S : pl.BK;
+    rows = (rows + pl.BK - 1) / pl.BK * pl.BK;
+    S = Me > 0 ? (Me + rows - 1) / rows : 1;
+    pl.S = (int)S;
+    pl.rows_per_split = (int)rows;
+    pl.bytes = S > 1 ? align_up((size_t)S * d->E * d->I * d->J * 4, 256) : 0;
+    return pl;
+}
+
+// ------------------------------------------------------------------------------ rows-GEMM dispatch
+template <class TT, int WES, bool GATHER, bool W_TRANS, int EPI>
+int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
+{
+    constexpr int BK = TT::ES == 4 ? 32 : 64;
+    const int Me = p.B * p.K;
+    if (Me == 0 || p.E == 0 || p.N == 0) return EGS_OK;
+    const int e_groups = ceil_div(p.E, 8);
+    if (p.N <= 64) {
+        constexpr int BM = 128, BN = 64;
+        p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
+        int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
+        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+        hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 4, 1, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
+                           dim3(kThreads), 0, s, p);
+    } else {
+        constexpr int BM = 128, BN = 128;
+        p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
+        int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
+        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+        hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
+                           dim3(kThreads), 0, s, p);
+    }
+    EGS_CHECK_LAUNCH("rows_gemm_kernel");
+    return EGS_OK;
+}
+
+template <class TT, bool GATHER, int EPI>
+int launch_rows_gemm_w(RowsGemmParams &p, bool w_trans, hipStream_t s)
+{
+    return w_trans ? launch_rows_gemm_cfg<TT, TT::ES, GATHER, true, EPI>(p, s)
+                   : launch_rows_gemm_cfg<TT, TT::ES, GATHER, false, EPI>(p, s);
+}
+
+template <bool GATHER, int EPI>
+int launch_rows_gemm(RowsGemmParams &p, int act_dtype, bool w_trans, hipStream_t s)
+{
+    switch (act_dtype) {
+    case EGS_F32: return launch_rows_gemm_w<ElemF32, GATHER, EPI>(p, w_trans, s);
+    case EGS_F16: return launch_rows_gemm_w<ElemF16, GATHER, EPI>(p, w_trans, s);
+    case EGS_BF16: return launch_rows_gemm_w<ElemBF16, GATHER, EPI>(p, w_trans, s);
+    default: return EGS_ERR_BAD_DTYPE;
+    }
+}
+
+// ------------------------------------------------------------------------------ implementations
+int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
+                     const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
+                     int w_layout, hipStream_t s)
+{
+    const int ES = elem_size(act_dtype), WES = elem_size(w_dtype);
+    RowsGemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y; p.w_scale = w_scale;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K;
+    p.R = d->I; p.N = d->J;
+    p.lda_b = ldx_b; p.lda_t = ldx_t;
+    p.ind_dtype = ind_dtype;
+    const bool w_trans = (w_layout == EGS_W_EIJ);       // [E,I,J]: the reduction index selects the row
+    p.a_vec = aligned_to(X, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
+    const int64_t w_row = w_trans ? d->J : d->I;
+    p.w_vec = WES == 1 ? (aligned_to(W, 8) && w_row % 8 == 0) : (aligned_to(W, 16) && (w_row * WES) % 16 == 0);
+    p.c_vec = aligned_to(Y, 16) && d->J % 4 == 0;
+    if (w_dtype == EGS_FP8_E4M3) {
+        return w_trans ? launch_rows_gemm_cfg<ElemBF16, 1, true, true, EPI_STORE>(p, s)
+                       : launch_rows_gemm_cfg<ElemBF16, 1, true, false, EPI_STORE>(p, s);
+    }
+    return launch_rows_gemm<true, EPI_STORE>(p, act_dtype, w_trans, s);
+}
+
+int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, void *workspace,
+                      const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode, hipStream_t s)
+{
+    const int ES = elem_size(act_dtype);
+    const size_t out_elems = (size_t)d->B * d->T * d->I;
+    if (out_elems == 0) return EGS_OK;
+    const ScatterPlan pl = plan_scatter(d, mode, act_dtype);
+    char *ws = (char *)workspace;
+    const int N = d->E * d->K;
+
+    RowsGemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)Y; p.W = (const char *)W; p.Ind = Ind;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K;
+    p.R = d->J; p.N = d->I;
+    p.ind_dtype = ind_dtype;
+    const bool w_trans = (w_layout == EGS_W_EJI);       // [E,J,I]: the reduction index j selects the row
+    p.a_vec = aligned_to(Y, 16) && ((int64_t)d->J * ES) % 16 == 0;
+    const int64_t w_row = w_trans ? d->I : d->J;
+    p.w_vec = aligned_to(W, 16) && (w_row * ES) % 16 == 0;
+
+    if (mode == EGS_SCATTER_ATOMIC) {
+        float *acc32 = act_dtype == EGS_F32 ? (float *)Out : (float *)(ws + pl.rows_at);
+        hipLaunchKernelGGL(fill_zero_f32_kernel, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s, acc32, out_elems,
+                           (int)aligned_to(acc32, 16));
+        EGS_CHECK_LAUNCH("fill_zero_f32_kernel");
+        p.C = (char *)acc32;
+        p.c_vec = 0;
+        int rc = launch_rows_gemm<false, EPI_ATOMIC_F32>(p, act_dtype, w_trans, s);
+        if (rc != EGS_OK) return rc;
+        if (act_dtype != EGS_F32) {
+            const int vec = (int)aligned_to(Out, 8);
+            if (act_dtype == EGS_BF16)
+                hipLaunchKernelGGL(downconvert_kernel<ElemBF16>, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s,
+                                   (const float *)acc32, (uint16_t *)Out, out_elems, vec);
+            else
+                hipLaunchKernelGGL(downconvert_kernel<ElemF16>, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s,
+                                   (const float *)acc32, (uint16_t *)Out, out_elems, vec);
+            EGS_CHECK_LAUNCH("downconvert_kernel");
+        }
+        return EGS_OK;
+    }
+
+    // deterministic: routing table, fp32 product rows, fixed-order reduction per token
+    int32_t *seg_off = (int32_t *)(ws + pl.seg_off_at);
+    int32_t *perm = (int32_t *)(ws + pl.perm_at);
+    int32_t *cnt = d->T > kCsrLdsTokens ? (int32_t *)(ws + pl.cnt_at) : nullptr;
+    float *rows = (float *)(ws + pl.rows_at);
+    const size_t lds = d->T > kCsrLdsTokens ? 0 : (size_t)d->T * 4;
+    hipLaunchKernelGGL(csr_build_kernel, dim3(d->B), dim3(kWave), lds, s, Ind, ind_dtype, d->T, N, seg_off, perm, cnt);
+    EGS_CHECK_LAUNCH("csr_build_kernel");
+    p.C = (char *)rows;
+    p.c_vec = d->I % 4 == 0;
+    int rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
+    if (rc != EGS_OK) return rc;
+    const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
+    const size_t items = (size_t)d->B * d->T * (vw4 ? d->I / 4 : d->I);
+    const int grid = grid_1d(items, 65536);
+#define EGS_SEGSUM(TT)                                                                                              \
+    do {                                                                                                            \
+        if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, 4>), dim3(grid), dim3(kThreads), 0, s, rows, seg_off,   \
+                                    perm, (char *)Out, d->B, d->T, N, d->I);                                        \
+        else hipLaunchKernelGGL((segment_sum_kernel<TT, 1>), dim3(grid), dim3(kThreads), 0, s, rows, seg_off, perm, \
+                                (char *)Out, d->B, d->T, N, d->I);                                                  \
+    } while (0)
+    if (act_dtype == EGS_F32) EGS_SEGSUM(ElemF32);
+    else if (act_dtype == EGS_F16) EGS_SEGSUM(ElemF16);
+    else EGS_SEGSUM(ElemBF16);
+#undef EGS_SEGSUM
+    EGS_CHECK_LAUNCH("segment_sum_kernel");
+    return EGS_OK;
+}
+
+int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
+            int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout, hipStream_t s)
+{
+    const size_t w_elems = (size_t)d->E * d->I * d->J;
+    if (w_elems == 0) return EGS_OK;
+    const int ES = elem_size(act_dtype), OES = elem_size(out_dtype);
+    const DwPlan pl = plan_dw(d, act_dtype);
+    DwParams p;
+    memset(&p, 0, sizeof(p));
+    p.Xs = (const char *)Xs; p.Ys = (const char *)Ys; p.Ind = Ind;
+    p.part = (float *)workspace; p.dW = (char *)dW;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.I = d->I; p.J = d->J;
+    p.ldx_b = ldx_b; p.ldx_t = ldx_t;
+    p.ind_dtype = ind_dtype;
+    p.x_vec = aligned_to(Xs, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
+    p.y_vec = aligned_to(Ys, 16) && ((int64_t)d->J * ES) % 16 == 0;
+    p.o_vec = aligned_to(dW, 16) && d->J % 4 == 0;
+    (void)OES;
+    p.i_tiles = pl.i_tiles; p.j_tiles = pl.j_tiles; p.S = pl.S; p.rows_per_split = pl.rows_per_split;
+    p.out_dtype = out_dtype; p.dw_layout = dw_layout;
+    const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.i_tiles * pl.j_tiles * pl.S;
+    if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+    switch (act_dtype) {
+    case EGS_F32: hipLaunchKernelGGL((dw_kernel<ElemF32, 128, 64, 32>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
+    case EGS_F16: hipLaunchKernelGGL((dw_kernel<ElemF16, 128, 64, 64>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
+    default: hipLaunchKernelGGL((dw_kernel<ElemBF16, 128, 64, 64>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
+    }
+    EGS_CHECK_LAUNCH("dw_kernel");
+    if (pl.S > 1) {
+        hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s, (const float *)workspace,
+                           (char *)dW, pl.S, d->E, d->I, d->J, out_dtype, dw_layout);
+        EGS_CHECK_LAUNCH("dw_reduce_kernel");
+    }
+    return EGS_OK;
+}
+
+// ------------------------------------------------------------------------------ validation
+int validate_gather(const void *X, const void *W, const void *Ind, const void *Y, const float *w_scale,
+                    const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
+                    int w_layout)
+{
+    int rc = check_dims(d);
+    if (rc != EGS_OK) return rc;
+    if (!act_dtype_ok(act_dtype) || !ind_dtype_ok(ind_dtype)) return EGS_ERR_BAD_DTYPE;
+    if (w_dtype == EGS_FP8_E4M3) {
+        if (act_dtype != EGS_BF16) return EGS_ERR_UNSUPPORTED;    // fp8 weights pair with bf16 activations
+        if (w_scale == nullptr) return EGS_ERR_NULL_POINTER;
+    } else if (w_dtype != act_dtype) {
+        return act_dtype_ok(w_dtype) ? EGS_ERR_UNSUPPORTED : EGS_ERR_BAD_DTYPE;
+    }
+    if (!layout_ok(w_layout)) return EGS_ERR_BAD_LAYOUT;
+    const size_t y_elems = (size_t)d->B * d->E * d->K * d->J;
+    if (y_elems == 0) return EGS_OK;
+    if (Y == nullptr || Ind == nullptr) return EGS_ERR_NULL_POINTER;
+    if (d->I > 0 && (X == nullptr || W == nullptr)) return EGS_ERR_NULL_POINTER;
+    if (d->I > 0 && d->T == 0) return EGS_OK;                      // every pick is out of range
+    if (ldx_t < d->I || (d->B > 1 && ldx_b < 0)) return EGS_ERR_BAD_STRIDE;
+    const int ES = elem_size(act_dtype);
+    if (!aligned_to(X, ES) || !aligned_to(Y, ES) || !aligned_to(W, elem_size(w_dtype))) return EGS_ERR_ALIGNMENT;
+    return EGS_OK;
+}
+
+int validate_scatter(const void *Y, const void *W, const void *Ind, const void *Out, const void *workspace,
+                     size_t workspace_bytes, const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode)
+{
+    int rc = check_dims(d);
+    if (rc != EGS_OK) return rc;
+    if (!act_dtype_ok(act_dtype) || !ind_dtype_ok(ind_dtype)) return EGS_ERR_BAD_DTYPE;
+    if (!layout_ok(w_layout)) return EGS_ERR_BAD_LAYOUT;
+    if (!mode_ok(mode)) return EGS_ERR_BAD_MODE;
+    const size_t out_elems = (size_t)d->B * d->T * d->I;
+    if (out_elems == 0) return EGS_OK;
+    if (Out == nullptr) return EGS_ERR_NULL_POINTER;
+    const size_t picks = (size_t)d->B * d->E * d->K;
+    if (picks > 0 && Ind == nullptr) return EGS_ERR_NULL_POINTER;
+    if (picks > 0 && d->J > 0 && (Y == nullptr || W == nullptr)) return EGS_ERR_NULL_POINTER;
+    const size_t need = plan_scatter(d, mode, act_dtype).bytes;
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return EGS_ERR_WORKSPACE;
+    if (need > 0 && !aligned_to(workspace, 256)) return EGS_ERR_ALIGNMENT;
+    const int ES = elem_size(act_dtype);
+    if (!aligned_to(Y, ES) || !aligned_to(Out, ES) || !aligned_to(W, ES)) return EGS_ERR_ALIGNMENT;
+    return EGS_OK;
+}
+
+int validate_dw(const void *Xs, const void *Ys, const void *Ind, const void *dW, const void *workspace,
+                size_t workspace_bytes, const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype,
+                int out_dtype, int ind_dtype, int dw_layout)
+{
+    int rc = check_dims(d);
+    if (rc != EGS_OK) return rc;
+    if (!act_dtype_ok(act_dtype) || !act_dtype_ok(out_dtype) || !ind_dtype_ok(ind_dtype)) return EGS_ERR_BAD_DTYPE;
+    if (!layout_ok(dw_layout)) return EGS_ERR_BAD_LAYOUT;
+    const size_t w_elems = (size_t)d->E * d->I * d->J;
+    if (w_elems == 0) return EGS_OK;
+    if (dW == nullptr) return EGS_ERR_NULL_POINTER;
+    const size_t picks = (size_t)d->B * d->K;
+    if (picks > 0 && (Xs == nullptr || Ys == nullptr || Ind == nullptr)) return EGS_ERR_NULL_POINTER;
+    if (picks > 0 && d->T > 0 && (ldx_t < d->I || (d->B > 1 && ldx_b < 0))) return EGS_ERR_BAD_STRIDE;
+    const size_t need = plan_dw(d, act_dtype).bytes;
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return EGS_ERR_WORKSPACE;
+    if (need > 0 && !aligned_to(workspace, 256)) return EGS_ERR_ALIGNMENT;
+    const int ES = elem_size(act_dtype);
+    if (!aligned_to(Xs, ES) || !aligned_to(Ys, ES) || !aligned_to(dW, elem_size(out_dtype))) return EGS_ERR_ALIGNMENT;
+    return EGS_OK;
+}
+
+}  // namespace
+
+// ================================================================================ C ABI
+extern "C" {
+
+int egs_abi_version(void) { return EGS_ABI_VERSION; }
+
+const char *egs_status_string(int status)
+{
+    switch (status) {
+    case EGS_OK: return "ok";
+    case EGS_ERR_NULL_POINTER: return "null pointer argument";
+    case EGS_ERR_BAD_SHAPE: return "negative or too large dimension";
+    case EGS_ERR_BAD_DTYPE: return "Unknown dtype";
+    case EGS_ERR_BAD_LAYOUT: return "unknown weight layout";
+    case EGS_ERR_BAD_MODE: return "unknown scatter mode";
+    case EGS_ERR_WORKSPACE: return "workspace missing or too small";
+    case EGS_ERR_ALIGNMENT: return "pointer not aligned to its element size (workspace: 256 bytes)";
+    case EGS_ERR_HIP: return "HIP runtime error";
+    case EGS_ERR_UNSUPPORTED: return "unsupported dtype combination";
+    case EGS_ERR_BAD_STRIDE: return "source stride smaller than its row";
+    default: return "unknown status";
+    }
+}
+
+const char *egs_last_hip_error(void) { return g_hip_error; }
+
+size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
+{
+    if (check_dims(d) != EGS_OK || !act_dtype_ok(act_dtype)) return 0;
+    if (!mode_ok(mode)) mode = EGS_SCATTER_DETERMINISTIC;
+    switch (op) {
+    case EGS_OP_GATHER_GEMM: return 0;
+    case EGS_OP_GEMM_SCATTER: return plan_scatter(d, mode, act_dtype).bytes;
+    case EGS_OP_DW: return plan_dw(d, act_dtype).bytes;
+    case EGS_OP_GATHER_BACKWARD: return plan_scatter(d, mode, act_dtype).bytes + plan_dw(d, act_dtype).bytes;
+    case EGS_OP_SCATTER_BACKWARD: return plan_dw(d, act_dtype).bytes;
+    default: return 0;
+    }
+}
+
+int egs_gather_gemm(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
+                    const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                    int act_dtype, int w_dtype, int ind_dtype, int w_layout, void *stream)
+{
+    int rc = validate_gather(X, W, Ind, Y, w_scale, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout);
+    if (rc != EGS_OK) return rc;
+    if ((size_t)d->B * d->E * d->K * d->J == 0) return EGS_OK;
+    return gather_gemm_impl(X, W, Ind, Y, w_scale, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout,
+                            (hipStream_t)stream);
+}
+
+int egs_gemm_scatter(const void *Y, const void *W, const void *Ind, void *Out,
+                     void *workspace, size_t workspace_bytes, const egs_dims *d,
+                     int act_dtype, int ind_dtype, int w_layout, int mode, void *stream)
+{
+    int rc = validate_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, act_dtype, ind_dtype, w_layout, mode);
+    if (rc != EGS_OK) return rc;
+    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, act_dtype, ind_dtype, w_layout, mode, (hipStream_t)stream);
+}
+
+int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
+           void *workspace, size_t workspace_bytes, const egs_dims *d,
+           int64_t ldx_b, int64_t ldx_t,
+           int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream)
+{
+    int rc = validate_dw(Xsrc, Ysrc, Ind, dW, workspace, workspace_bytes, d, ldx_b, ldx_t, act_dtype, out_dtype,
+                         ind_dtype, dw_layout);
+    if (rc != EGS_OK) return rc;
+    return dw_impl(Xsrc, Ysrc, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout,
+                   (hipStream_t)stream);
+}
+
+int egs_expert_gather_forward(const void *X, const void *W, const void *Ind, void *Y,
+                              const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                              int dtype, int ind_dtype, void *stream)
+{
+    return egs_gather_gemm(X, W, Ind, Y, nullptr, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, stream);
+}
+
+int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, const void *grad_Y,
+                               void *grad_X, void *grad_W,
+                               void *workspace, size_t workspace_bytes, const egs_dims *d,
+                               int64_t ldx_b, int64_t ldx_t,
+                               int dtype, int ind_dtype, int mode, void *stream)
+{
+    int rc = check_dims(d);
+    if (rc != EGS_OK) return rc;
+    if (!act_dtype_ok(dtype)) return EGS_ERR_BAD_DTYPE;
+    if (!mode_ok(mode)) return EGS_ERR_BAD_MODE;
+    const size_t ws_scatter = plan_scatter(d, mode, dtype).bytes;
+    const size_t ws_dw = plan_dw(d, dtype).bytes;
+    if (ws_scatter + ws_dw > 0 && (workspace == nullptr || workspace_bytes < ws_scatter + ws_dw)) return EGS_ERR_WORKSPACE;
+    // validate both halves before enqueuing anything
+    rc = validate_scatter(grad_Y, W, Ind, grad_X, workspace, ws_scatter, d, dtype, ind_dtype, EGS_W_EIJ, mode);
+    if (rc != EGS_OK) return rc;
+    void *ws2 = workspace ? (char *)workspace + ws_scatter : nullptr;
+    rc = validate_dw(X, grad_Y, Ind, grad_W, ws2, ws_dw, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ);
+    if (rc != EGS_OK) return rc;
+    // grad_X[b,t,i] = sum_picks sum_j grad_Y[b,e,k,j] * W[e,i,j]
+    rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, (hipStream_t)stream);
+    if (rc != EGS_OK) return rc;
+    return dw_impl(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, (hipStream_t)stream);
+}
+
+int egs_expert_scatter_forward(const void *Y, const void *W, const void *Ind, void *Out,
+                               void *workspace, size_t workspace_bytes, const egs_dims *d,
+                               int dtype, int ind_dtype, int mode, void *stream)
+{
+    return egs_gemm_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, dtype, ind_dtype, EGS_W_EJI, mode, stream);
+}
+
+int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, const void *grad_Out,
+                                void *grad_Y, void *grad_W,
+                                void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                int64_t ldg_b, int64_t ldg_t,
+                                int dtype, int ind_dtype, void *stream)
+{
+    int rc = validate_gather(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI);
+    if (rc != EGS_OK) return rc;
+    rc = validate_dw(grad_Out, Y, Ind, grad_W, workspace, workspace_bytes, d, ldg_b, ldg_t, dtype, dtype, ind_dtype,
+                     EGS_W_EJI);
+    if (rc != EGS_OK) return rc;
+    // grad_Y[b,e,k,j] = sum_i grad_Out[b,Ind,i] * W[e,j,i]
+    if ((size_t)d->B * d->E * d->K * d->J > 0) {
+        rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI,
+                              (hipStream_t)stream);
+        if (rc != EGS_OK) return rc;
+    }
+    // grad_W[e,j,i] = sum_{b,k} grad_Out[b,Ind,i] * Y[b,e,k,j]
+    return dw_impl(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI,
+                   (hipStream_t)stream);
+}
+
+int egs_validate_indices(const void *Ind, int ind_dtype, int64_t n, int32_t T, int32_t *d_bad_count, void *stream)
+{
+    if (n < 0) return EGS_ERR_BAD_SHAPE;
+    if (!ind_dtype_ok(ind_dtype)) return EGS_ERR_BAD_DTYPE;
+    if (n == 0) return EGS_OK;
+    if (Ind == nullptr || d_bad_count == nullptr) return EGS_ERR_NULL_POINTER;
+    hipLaunchKernelGGL(validate_indices_kernel, dim3(grid_1d((size_t)n, 1024)), dim3(kThreads), 0, (hipStream_t)stream,
+                       Ind, ind_dtype, n, T, d_bad_count);
+    EGS_CHECK_LAUNCH("validate_indices_kernel");
+    return EGS_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,271 @@
+// Per-expert "rows x weight" product with an index on one side:
+//
+//   gather   C[m, n] = sum_r A[b, Ind[m], r] * Wt(n, r)     rows of A fetched through Ind, C dense
+//   scatter  C[b, Ind[m], n] += sum_r A[m, r] * Wt(n, r)    A dense, rows of C addressed through Ind
+//
+// where m = b*K + k enumerates the picks of one expert e.  One workgroup owns a BM x BN tile
+// of one expert's product, stages BK-wide slabs of both operands in K-major swizzled LDS
+// tiles (register prefetch of the next slab overlaps the MFMAs of the current one) and runs
+// 16x16 MFMA tiles on 4 wavefronts.
+//
+// Replaces the reference's expert_gather_kernel (egs/triton_kernels.py:49-143) and
+// expert_scatter_kernel (:156-247).  Unlike those, the M dimension of a tile is the picks of
+// one expert (not batch rows of one (e,k)), so W[e] is read once per tile instead of once
+// per pick.
+#pragma once
+#include "egs_device.h"
+
+namespace egs {
+
+enum : int { EPI_STORE = 0, EPI_STORE_F32 = 1, EPI_ATOMIC_F32 = 2 };
+
+struct RowsGemmParams {
+    const char *A;          // gather: [B,T,R] source;  scatter: [B,E,K,R] dense rows
+    const char *W;          // [E,R,N] (W_TRANS) or [E,N,R]
+    const void *Ind;        // [B,E,K]
+    char *C;                // gather: [B,E,K,N];  scatter: fp32 [B,E,K,N] rows or fp32 [B,T,N] accumulator
+    const float *w_scale;   // [E,N] or nullptr
+    int32_t B, T, E, K;
+    int32_t R, N;           // reduction length, output columns
+    int64_t lda_b, lda_t;   // element strides of the [B,T,R] source (gather)
+    int32_t ind_dtype;
+    int32_t a_vec, w_vec, c_vec;   // 1 when 16-byte accesses are safe on that tensor
+    int32_t m_tiles, n_tiles;
+};
+
+template <class TT, int WES, int BM, int BN, int BK, int WM, int WN, bool GATHER, bool W_TRANS, int EPI>
+__global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
+{
+    constexpr int ES = TT::ES, VEC = TT::VEC;
+    constexpr int CH = BK / VEC;                 // chunks per LDS row
+    constexpr int KSTEPS = CH / 4;               // MFMA chunk steps per slab
+    constexpr bool SWAP = (EPI == EPI_ATOMIC_F32);   // atomics want consecutive n across lanes
+    constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
+    constexpr bool W_FP8 = (WES == 1);
+    static_assert(WM * WN == kThreads / kWave, "wave grid must cover the workgroup");
+    static_assert(BM <= kThreads, "row bookkeeping uses one thread per tile row");
+    static_assert((BM * CH) % kThreads == 0 && kThreads % CH == 0, "M loader mapping");
+    static_assert(!W_FP8 || TT::ES == 2, "fp8 weights are widened to bf16");
+
+    __shared__ __attribute__((aligned(16))) char smem_m[BM * BK * ES];
+    __shared__ __attribute__((aligned(16))) char smem_n[BN * BK * ES];
+    __shared__ int64_t a_off[BM];
+    __shared__ int64_t c_off[BM];
+
+    int e, tile;
+    if (!decode_expert_tile((int)blockIdx.x, p.m_tiles * p.n_tiles, p.E, e, tile)) return;
+    const int mt = tile / p.n_tiles, nt = tile - mt * p.n_tiles;
+    const int m0 = mt * BM, n0 = nt * BN;
+    const int tid = (int)threadIdx.x;
+    const int R = p.R, N = p.N;
+    const char *We = p.W + (size_t)e * R * N * WES;
+    const bool w_vec = p.w_vec != 0, a_vec = p.a_vec != 0;
+
+    // ---------------- weight-side loader
+    constexpr int NVN = (BN * CH + kThreads - 1) / kThreads;            // K-major: chunks per thread
+    constexpr int KB = BK / VEC, NBK = BN / VEC;                        // transposed: VEC x VEC blocks
+    constexpr int NBL = (KB * NBK + kThreads - 1) / kThreads;
+    u32x4 nreg[W_TRANS ? NBL * VEC : NVN];
+
+    auto issue_n = [&](int kt) {
+        if constexpr (!W_TRANS) {
+#pragma unroll
+            for (int i = 0; i < NVN; ++i) {
+                int v = tid + i * kThreads;
+                int row = v / CH, c = v % CH;
+                int n = n0 + row;
+                const char *ptr = (v < BN * CH && n < N) ? We + (size_t)n * R * WES : nullptr;
+                if constexpr (W_FP8) nreg[i] = load_chunk_fp8_as_bf16(ptr, kt * BK + c * VEC, R, w_vec);
+                else nreg[i] = load_chunk<ES>(ptr, kt * BK + c * VEC, R, w_vec);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NBL; ++i) {
+                int blk = tid + i * kThreads;
+                int kb = blk / NBK, nb = blk % NBK;
+#pragma unroll
+                for (int r = 0; r < VEC; ++r) {
+                    int rr = kt * BK + kb * VEC + r;
+                    const char *ptr = (blk < KB * NBK && rr < R) ? We + (size_t)rr * N * WES : nullptr;
+                    if constexpr (W_FP8) nreg[i * VEC + r] = load_chunk_fp8_as_bf16(ptr, n0 + nb * VEC, N, w_vec);
+                    else nreg[i * VEC + r] = load_chunk<ES>(ptr, n0 + nb * VEC, N, w_vec);
+                }
+            }
+        }
+    };
+    auto commit_n = [&]() {
+        u32x4 *tile_n = reinterpret_cast<u32x4 *>(smem_n);
+        if constexpr (!W_TRANS) {
+#pragma unroll
+            for (int i = 0; i < NVN; ++i) {
+                int v = tid + i * kThreads;
+                if (v < BN * CH) tile_n[tile_chunk_index<CH>(v / CH, v % CH)] = nreg[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NBL; ++i) {
+                int blk = tid + i * kThreads;
+                int kb = blk / NBK, nb = blk % NBK;
+                if (blk < KB * NBK) {
+                    u32x4 in[VEC], out[VEC];
+#pragma unroll
+                    for (int r = 0; r < VEC; ++r) in[r] = nreg[i * VEC + r];
+                    if constexpr (VEC == 8) transpose8x8_16b(in, out); else transpose4x4_32b(in, out);
+#pragma unroll
+                    for (int c = 0; c < VEC; ++c) tile_n[tile_chunk_index<CH>(nb * VEC + c, kb)] = out[c];
+                }
+            }
+        }
+    };
+
+    issue_n(0);     // does not depend on Ind: overlap with the index fetch below
+
+    // ---------------- per-row bookkeeping: where each tile row reads from / writes to
+    const int Me = p.B * p.K;
+    if (tid < BM) {
+        int m = m0 + tid;
+        int64_t ao = -1, co = -1;
+        if (m < Me) {
+            int b = m / p.K, k = m - b * p.K;
+            int64_t pick = ((int64_t)b * p.E + e) * p.K + k;
+            if constexpr (GATHER) {
+                int32_t t = load_token(p.Ind, p.ind_dtype, pick, p.T);
+                ao = t < 0 ? -1 : (int64_t)b * p.lda_b + (int64_t)t * p.lda_t;
+                co = pick * N;
+            } else {
+                ao = pick * R;
+                if constexpr (EPI == EPI_ATOMIC_F32) {
+                    int32_t t = load_token(p.Ind, p.ind_dtype, pick, p.T);
+                    co = t < 0 ? -1 : ((int64_t)b * p.T + t) * N;
+                } else {
+                    co = pick * N;
+                }
+            }
+        }
+        a_off[tid] = ao;
+        c_off[tid] = co;
+    }
+    __syncthreads();
+
+    // ---------------- row-side loader (K-major source rows)
+    constexpr int NVM = BM * CH / kThreads;
+    const int mc = tid % CH;
+    const char *mrow[NVM];
+    u32x4 mreg[NVM];
+#pragma unroll
+    for (int i = 0; i < NVM; ++i) {
+        int64_t ao = a_off[tid / CH + i * (kThreads / CH)];
+        mrow[i] = ao < 0 ? nullptr : p.A + ao * ES;
+    }
+    auto issue_m = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < NVM; ++i) mreg[i] = load_chunk<ES>(mrow[i], kt * BK + mc * VEC, R, a_vec);
+    };
+    auto commit_m = [&]() {
+        u32x4 *tile_m = reinterpret_cast<u32x4 *>(smem_m);
+#pragma unroll
+        for (int i = 0; i < NVM; ++i) tile_m[tile_chunk_index<CH>(tid / CH + i * (kThreads / CH), mc)] = mreg[i];
+    };
+    issue_m(0);
+
+    // ---------------- MFMA main loop
+    const int lane = tid & 63, wave = tid >> 6;
+    const int a = lane & 15, g = lane >> 4;
+    const int wave_m0 = (wave / WN) * (BM / WM), wave_n0 = (wave % WN) * (BN / WN);
+    f32x4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // fragment rows.  Without SWAP the weight side supplies the accumulator's row axis and its
+    // rows are relabelled so that one lane ends up with 4*TN consecutive output columns.
+    int mrow_l[TM], nrow_l[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) mrow_l[i] = wave_m0 + i * 16 + a;
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+        nrow_l[j] = SWAP ? wave_n0 + j * 16 + a : wave_n0 + (a >> 2) * (4 * TN) + j * 4 + (a & 3);
+
+    const int nk = (R + BK - 1) / BK;
+    for (int kt = 0; kt < nk; ++kt) {
+        commit_m();
+        commit_n();
+        __syncthreads();
+        if (kt + 1 < nk) { issue_n(kt + 1); issue_m(kt + 1); }
+        const u32x4 *tile_m = reinterpret_cast<const u32x4 *>(smem_m);
+        const u32x4 *tile_n = reinterpret_cast<const u32x4 *>(smem_n);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 mf[TM], nf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) mf[i] = tile_m[tile_chunk_index<CH>(mrow_l[i], ks * 4 + g)];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) nf[j] = tile_n[tile_chunk_index<CH>(nrow_l[j], ks * 4 + g)];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (SWAP) mma_chunk<TT>(acc[i][j], mf[i], nf[j]);
+                    else mma_chunk<TT>(acc[i][j], nf[j], mf[i]);
+                }
+        }
+        __syncthreads();
+    }
+
+    // ---------------- epilogue
+    if constexpr (!SWAP) {
+        constexpr int OES = (EPI == EPI_STORE_F32) ? 4 : ES;
+        const bool c_vec = p.c_vec != 0;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            int64_t co = c_off[wave_m0 + i * 16 + a];
+            if (co < 0) continue;
+            char *crow = p.C + co * OES;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                int n = n0 + wave_n0 + g * (4 * TN) + j * 4;
+                if (n >= N) continue;
+                f32x4 v = acc[i][j];
+                if (p.w_scale != nullptr) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (n + r < N) v[r] *= p.w_scale[(size_t)e * N + n + r];
+                }
+                if (c_vec && n + 4 <= N) {
+                    if constexpr (OES == 4) {
+                        *reinterpret_cast<f32x4 *>(crow + (size_t)n * 4) = v;
+                    } else {
+                        u32x2 w;
+                        w[0] = f32_to_elem_bits<TT>(v[0]) | (f32_to_elem_bits<TT>(v[1]) << 16);
+                        w[1] = f32_to_elem_bits<TT>(v[2]) | (f32_to_elem_bits<TT>(v[3]) << 16);
+                        *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = w;
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (n + r >= N) continue;
+                        if constexpr (OES == 4) reinterpret_cast<float *>(crow)[n + r] = v[r];
+                        else reinterpret_cast<uint16_t *>(crow)[n + r] = (uint16_t)f32_to_elem_bits<TT>(v[r]);
+                    }
+                }
+            }
+        }
+    } else {
+        float *cbase = reinterpret_cast<float *>(p.C);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                int64_t co = c_off[wave_m0 + i * 16 + g * 4 + r];
+                if (co < 0) continue;
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    int n = n0 + wave_n0 + j * 16 + a;
+                    if (n < N) unsafeAtomicAdd(cbase + co + n, acc[i][j][r]);
+                }
+            }
+    }
+}
+
+}  // namespace egs

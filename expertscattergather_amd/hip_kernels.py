@@ -1,0 +1,351 @@
+"""Launchers and autograd Functions of the fused expert gather / scatter-with-linear path.
+
+Same surface as the reference's ``egs/triton_kernels.py``: ``create_kernels()`` binds the four
+module-level callables
+
+    expert_gather_forward_call  (X[B,T,I], W[E,I,J], Ind[B,E,K], out_dtype)          -> Y[B,E,K,J]
+    expert_gather_backward_call (X, W, Ind, grad_output[B,E,K,J], dtype)             -> (grad_X, grad_W)
+    expert_scatter_forward_call (Y[B,E,K,J], W[E,J,I], Ind[B,E,K], T, out_dtype)     -> X[B,T,I]
+    expert_scatter_backward_call(Y, W, Ind, grad_X[B,T,I], dtype)                    -> (grad_Y, grad_W)
+
+(reference egs/triton_kernels.py:26-29, :361-578) and ``ExpertGatherFunction`` /
+``ExpertScatterFunction`` (reference :581-639) call them.  Here the callables allocate the
+outputs with torch and hand raw device pointers to the HIP library through its C ABI on the
+current stream; they are registered as ``torch.library`` custom ops with fake implementations
+so that ``torch.compile`` can trace through them.
+"""
+from __future__ import annotations
+
+import os
+import threading
+
+import torch
+
+from . import _abi
+
+__all__ = [
+    "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
+    "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "validate_indices",
+]
+
+OP_NAMESPACE = "egs_amd"
+
+
+def dtype_to_type_id(dtype: torch.dtype) -> int:
+    """float32 -> 0, float16 -> 1, bfloat16 -> 2 (reference egs/triton_kernels.py:15-23)."""
+    if dtype == torch.float32:
+        return _abi.F32
+    if dtype == torch.float16:
+        return _abi.F16
+    if dtype == torch.bfloat16:
+        return _abi.BF16
+    raise ValueError("Unknown dtype")
+
+
+_IND_IDS = {torch.int16: _abi.IND_I16, torch.int32: _abi.IND_I32, torch.int64: _abi.IND_I64, torch.uint8: _abi.IND_U8}
+
+
+def _ind_type_id(Ind: torch.Tensor) -> int:
+    try:
+        return _IND_IDS[Ind.dtype]
+    except KeyError:
+        raise ValueError(f"Ind must be uint8, int16, int32 or int64, got {Ind.dtype}") from None
+
+
+# ------------------------------------------------------------------------------ scatter mode
+_MODES = {"deterministic": _abi.SCATTER_DETERMINISTIC, "atomic": _abi.SCATTER_ATOMIC}
+_scatter_mode = os.environ.get("EGS_SCATTER_MODE", "deterministic").lower()
+if _scatter_mode not in _MODES:
+    raise ValueError(f"EGS_SCATTER_MODE must be one of {sorted(_MODES)}, got {_scatter_mode!r}")
+
+
+def set_scatter_mode(mode: str) -> None:
+    """'deterministic' (fixed summation order, bitwise reproducible) or 'atomic' (fp32 atomics)."""
+    global _scatter_mode
+    mode = mode.lower()
+    if mode not in _MODES:
+        raise ValueError(f"scatter mode must be one of {sorted(_MODES)}, got {mode!r}")
+    _scatter_mode = mode
+
+
+def get_scatter_mode() -> str:
+    return _scatter_mode
+
+
+# ------------------------------------------------------------------------------ plumbing
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(
+                "the egs HIP kernels need tensors on an AMD GPU (HIP device), got a tensor on "
+                f"'{t.device}'; there is no CPU fallback")
+        if t.device != dev:
+            raise RuntimeError(f"all tensors must be on the same device, got {dev} and {t.device}")
+    return dev
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+_workspaces: dict = {}
+
+
+def _workspace(dev: torch.device, nbytes: int):
+    """Scratch buffer per (device, stream), grown on demand; returns (ptr, nbytes)."""
+    if nbytes == 0:
+        return None, 0
+    key = (dev.index, _stream_ptr(dev))
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=dev)
+        _workspaces[key] = buf
+    return buf.data_ptr(), buf.numel()
+
+
+def _rows_source(X: torch.Tensor):
+    """[B,T,I] tensor -> (tensor with unit inner stride, batch stride, token stride)."""
+    if X.stride(2) != 1 and X.shape[2] > 1:
+        X = X.contiguous()
+    B, T, I = X.shape
+    ld_t = X.stride(1) if T > 1 else max(I, 1)
+    ld_b = X.stride(0) if B > 1 else ld_t * max(T, 1)
+    if ld_t < I or ld_b < 0:
+        X = X.contiguous()
+        ld_t, ld_b = I, T * I
+    return X, ld_b, ld_t
+
+
+def _check_shapes(X3, W, Ind, Y4, w_is_eij: bool):
+    """Common shape checks; X3 is the [B,T,I] side, Y4 the [B,E,K,J] side (either may be None)."""
+    if W.dim() != 3 or Ind.dim() != 3:
+        raise ValueError("W must be 3-D and Ind must be [B,E,K]")
+    E = W.shape[0]
+    I, J = (W.shape[1], W.shape[2]) if w_is_eij else (W.shape[2], W.shape[1])
+    B, E2, K = Ind.shape
+    if E2 != E:
+        raise ValueError(f"Ind has {E2} experts but W has {E}")
+    if X3 is not None:
+        if X3.dim() != 3 or X3.shape[0] != B or X3.shape[2] != I:
+            raise ValueError(f"expected a [B={B},T,I={I}] tensor, got {tuple(X3.shape)}")
+    if Y4 is not None:
+        if Y4.dim() != 4 or tuple(Y4.shape) != (B, E, K, J):
+            raise ValueError(f"expected a [B={B},E={E},K={K},J={J}] tensor, got {tuple(Y4.shape)}")
+    return B, E, K, I, J
+
+
+def _same_dtype(*tensors):
+    dt = tensors[0].dtype
+    for t in tensors[1:]:
+        if t.dtype != dt:
+            raise ValueError(f"activations and weights must share one dtype, got {dt} and {t.dtype}")
+    return dtype_to_type_id(dt)
+
+
+# ------------------------------------------------------------------------------ the four launchers
+def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    dtype_to_type_id(out_dtype)
+    dev = _require_gpu(X, W, Ind)
+    B, E, K, I, J = _check_shapes(X, W, Ind, None, True)
+    dt = _same_dtype(X, W)
+    X, ld_b, ld_t = _rows_source(X)
+    W = W.contiguous(); Ind = Ind.contiguous()
+    Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
+    d = _abi.Dims(B, X.shape[1], E, K, I, J)
+    with torch.cuda.device(dev):
+        rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
+                                                  ld_b, ld_t, dt, _ind_type_id(Ind), _stream_ptr(dev))
+    _abi.check(rc, "expert_gather_forward_call")
+    return Y
+
+
+def _gather_backward_impl(X, W, Ind, grad_output, dtype):
+    dtype_to_type_id(dtype)
+    dev = _require_gpu(X, W, Ind, grad_output)
+    B, E, K, I, J = _check_shapes(X, W, Ind, grad_output, True)
+    dt = _same_dtype(X, W, grad_output)
+    X, ld_b, ld_t = _rows_source(X)
+    W = W.contiguous(); Ind = Ind.contiguous(); grad_output = grad_output.contiguous()
+    T = X.shape[1]
+    grad_X = torch.empty((B, T, I), device=dev, dtype=X.dtype)
+    grad_W = torch.empty((E, I, J), device=dev, dtype=W.dtype)
+    d = _abi.Dims(B, T, E, K, I, J)
+    mode = _MODES[_scatter_mode]
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt))
+        rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
+                                                   grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
+                                                   dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+    _abi.check(rc, "expert_gather_backward_call")
+    return grad_X, grad_W
+
+
+def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
+    dtype_to_type_id(out_dtype)
+    dev = _require_gpu(Y, W, Ind)
+    B, E, K, I, J = _check_shapes(None, W, Ind, Y, False)
+    dt = _same_dtype(Y, W)
+    T = int(T)
+    if T < 0:
+        raise ValueError("T must be non-negative")
+    Y = Y.contiguous(); W = W.contiguous(); Ind = Ind.contiguous()
+    out = torch.empty((B, T, I), device=dev, dtype=Y.dtype)
+    d = _abi.Dims(B, T, E, K, I, J)
+    mode = _MODES[_scatter_mode]
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt))
+        rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
+                                                   ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+    _abi.check(rc, "expert_scatter_forward_call")
+    return out
+
+
+def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
+    dtype_to_type_id(dtype)
+    dev = _require_gpu(Y, W, Ind, grad_X)
+    B, E, K, I, J = _check_shapes(grad_X, W, Ind, Y, False)
+    dt = _same_dtype(Y, W, grad_X)
+    grad_X, ld_b, ld_t = _rows_source(grad_X)
+    Y = Y.contiguous(); W = W.contiguous(); Ind = Ind.contiguous()
+    T = grad_X.shape[1]
+    grad_Y = torch.empty((B, E, K, J), device=dev, dtype=Y.dtype)
+    grad_W = torch.empty((E, J, I), device=dev, dtype=W.dtype)
+    d = _abi.Dims(B, T, E, K, I, J)
+    with torch.cuda.device(dev):
+        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, d, dt))
+        rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
+                                                    grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
+                                                    dt, _ind_type_id(Ind), _stream_ptr(dev))
+    _abi.check(rc, "expert_scatter_backward_call")
+    return grad_Y, grad_W
+
+
+# module globals, bound by create_kernels() (reference egs/triton_kernels.py:26-29)
+expert_gather_forward_call = None
+expert_gather_backward_call = None
+expert_scatter_forward_call = None
+expert_scatter_backward_call = None
+_create_lock = threading.Lock()
+
+
+def create_kernels() -> None:
+    """Register the four ops once per process and bind the module-level callables.
+
+    Counterpart of reference egs/triton_kernels.py:32-578; here it only defines the
+    ``torch.library`` ops (nothing is compiled at run time) and is safe to call from several
+    threads."""
+    global expert_gather_forward_call, expert_gather_backward_call
+    global expert_scatter_forward_call, expert_scatter_backward_call
+    if expert_scatter_backward_call is not None:
+        return
+    with _create_lock:
+        if expert_scatter_backward_call is not None:
+            return
+        ns = OP_NAMESPACE
+        lib = torch.library.Library(ns, "DEF")
+        lib.define("expert_gather_forward_call_fn(Tensor X, Tensor W, Tensor Ind, ScalarType out_dtype) -> Tensor")
+        lib.define("expert_gather_backward_call_fn(Tensor X, Tensor W, Tensor Ind, Tensor grad_output, "
+                   "ScalarType out_dtype) -> (Tensor, Tensor)")
+        lib.define("expert_scatter_forward_call_fn(Tensor Y, Tensor W, Tensor Ind, int T, ScalarType out_dtype) -> Tensor")
+        lib.define("expert_scatter_backward_call_fn(Tensor Y, Tensor W, Tensor Ind, Tensor grad_X, "
+                   "ScalarType out_dtype) -> (Tensor, Tensor)")
+        lib.impl("expert_gather_forward_call_fn", _gather_forward_impl, "CompositeExplicitAutograd")
+        lib.impl("expert_gather_backward_call_fn", _gather_backward_impl, "CompositeExplicitAutograd")
+        lib.impl("expert_scatter_forward_call_fn", _scatter_forward_impl, "CompositeExplicitAutograd")
+        lib.impl("expert_scatter_backward_call_fn", _scatter_backward_impl, "CompositeExplicitAutograd")
+
+        @torch.library.register_fake(f"{ns}::expert_gather_forward_call_fn", lib=lib)
+        def _(X, W, Ind, out_dtype):
+            return X.new_empty((X.shape[0], W.shape[0], Ind.shape[2], W.shape[2]))
+
+        @torch.library.register_fake(f"{ns}::expert_gather_backward_call_fn", lib=lib)
+        def _(X, W, Ind, grad_output, out_dtype):
+            return torch.empty_like(X, memory_format=torch.contiguous_format), torch.empty_like(
+                W, memory_format=torch.contiguous_format)
+
+        @torch.library.register_fake(f"{ns}::expert_scatter_forward_call_fn", lib=lib)
+        def _(Y, W, Ind, T, out_dtype):
+            return Y.new_empty((Y.shape[0], T, W.shape[2]))
+
+        @torch.library.register_fake(f"{ns}::expert_scatter_backward_call_fn", lib=lib)
+        def _(Y, W, Ind, grad_X, out_dtype):
+            return torch.empty_like(Y, memory_format=torch.contiguous_format), torch.empty_like(
+                W, memory_format=torch.contiguous_format)
+
+        create_kernels._lib = lib        # keep the registration alive
+        ops = getattr(torch.ops, ns)
+        expert_gather_forward_call = ops.expert_gather_forward_call_fn
+        expert_gather_backward_call = ops.expert_gather_backward_call_fn
+        expert_scatter_forward_call = ops.expert_scatter_forward_call_fn
+        expert_scatter_backward_call = ops.expert_scatter_backward_call_fn
+
+
+# ------------------------------------------------------------------------------ autograd Functions
+class ExpertGatherFunction(torch.autograd.Function):
+    """Y[b,e,k,j] = sum_i X[b, Ind[b,e,k], i] * W[e,i,j]   (reference egs/triton_kernels.py:581-608)."""
+
+    @staticmethod
+    def forward(ctx, X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, out_type=torch.float32):
+        create_kernels()
+        ctx.save_for_backward(X, W, Ind)
+        ctx.dtype = out_type
+        return expert_gather_forward_call(X, W, Ind, out_type)
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        X, W, Ind = ctx.saved_tensors
+        grad_X, grad_W = expert_gather_backward_call(X, W, Ind, grad_output, ctx.dtype)
+        return grad_X, grad_W, None, None
+
+
+class ExpertScatterFunction(torch.autograd.Function):
+    """X[b,t,i] = sum_{e,k: Ind[b,e,k]=t} sum_j Y[b,e,k,j] * W[e,j,i]   (reference egs/triton_kernels.py:610-639)."""
+
+    @staticmethod
+    def forward(ctx, Y: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, T: int, out_type=torch.float32):
+        create_kernels()
+        ctx.save_for_backward(Y, W, Ind)
+        ctx.dtype = out_type
+        return expert_scatter_forward_call(Y, W, Ind, T, out_type)
+
+    @staticmethod
+    def backward(ctx, grad_X: torch.Tensor):
+        Y, W, Ind = ctx.saved_tensors
+        grad_Y, grad_W = expert_scatter_backward_call(Y, W, Ind, grad_X, ctx.dtype)
+        return grad_Y, grad_W, None, None
+
+
+# ------------------------------------------------------------------------------ extras (not in the reference)
+def expert_gather_fp8w_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, Ind: torch.Tensor) -> torch.Tensor:
+    """Inference-only gather with fp8 weights: Y = X[b,Ind] . (Wq[e] * scale[e, None, :]).
+
+    X is bfloat16 [B,T,I]; Wq is float8_e4m3fn [E,I,J]; scale is float32 [E,J]."""
+    dev = _require_gpu(X, Wq, scale, Ind)
+    if X.dtype != torch.bfloat16 or Wq.dtype != torch.float8_e4m3fn or scale.dtype != torch.float32:
+        raise ValueError("fp8-weight gather needs bfloat16 X, float8_e4m3fn W and float32 scale")
+    B, E, K, I, J = _check_shapes(X, Wq, Ind, None, True)
+    if tuple(scale.shape) != (E, J):
+        raise ValueError(f"scale must be [E={E},J={J}], got {tuple(scale.shape)}")
+    X, ld_b, ld_t = _rows_source(X)
+    Wq = Wq.contiguous(); scale = scale.contiguous(); Ind = Ind.contiguous()
+    Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
+    d = _abi.Dims(B, X.shape[1], E, K, I, J)
+    with torch.cuda.device(dev):
+        rc = _abi.lib().egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), scale.data_ptr(), d,
+                                        ld_b, ld_t, _abi.BF16, _abi.FP8_E4M3, _ind_type_id(Ind), _abi.W_EIJ,
+                                        _stream_ptr(dev))
+    _abi.check(rc, "expert_gather_fp8w_forward")
+    return Y
+
+
+def validate_indices(Ind: torch.Tensor, T: int) -> int:
+    """Number of entries of Ind outside [0, T) (synchronises; debugging aid)."""
+    dev = _require_gpu(Ind)
+    Ind = Ind.contiguous()
+    bad = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _abi.lib().egs_validate_indices(Ind.data_ptr(), _ind_type_id(Ind), Ind.numel(), int(T), bad.data_ptr(),
+                                             _stream_ptr(dev))
+    _abi.check(rc, "validate_indices")
+    return int(bad.item())

@@ -1,0 +1,171 @@
+/*
+ * egs_hip.h -- C ABI of the MI355X (gfx950) fused expert gather / scatter-with-linear library.
+ *
+ * The reference reaches its device code through four Python callables bound in module
+ * globals (reference egs/triton_kernels.py:26-29, bound at :569-578) which launch three
+ * Triton kernels (:49-143 gather, :156-247 scatter, :261-356 dW).  This header is what a
+ * binding of that surface sees instead: plain device pointers, sizes and enums.
+ *
+ * Conventions for every entry point
+ *   - returns EGS_OK (0) or a negative egs_status; never throws, never synchronises;
+ *   - all tensor pointers are device pointers, borrowed until the enqueued work completes;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = default stream);
+ *   - arguments are validated before any HIP call, so bad arguments are reported even on a
+ *     host without a GPU;
+ *   - no device memory is allocated: scratch is a caller-provided workspace whose size comes
+ *     from egs_workspace_bytes();
+ *   - tensors are dense row-major ([B,T,I] sources may carry explicit batch/token strides,
+ *     inner stride 1);  Ind is [B,E,K] of int16/int32/int64/uint8 and is never written;
+ *   - a pick whose index is outside [0,T) contributes nothing (gather writes a zero row,
+ *     scatter and dW skip it); egs_validate_indices() reports such picks.
+ */
+#ifndef EGS_HIP_H
+#define EGS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EGS_ABI_VERSION 1
+
+typedef enum egs_status {
+    EGS_OK = 0,
+    EGS_ERR_NULL_POINTER = -1,
+    EGS_ERR_BAD_SHAPE = -2,
+    EGS_ERR_BAD_DTYPE = -3,     /* counterpart of ValueError("Unknown dtype"), reference egs/triton_kernels.py:23 */
+    EGS_ERR_BAD_LAYOUT = -4,
+    EGS_ERR_BAD_MODE = -5,
+    EGS_ERR_WORKSPACE = -6,     /* workspace missing or smaller than egs_workspace_bytes() */
+    EGS_ERR_ALIGNMENT = -7,
+    EGS_ERR_HIP = -8,           /* a HIP runtime call failed; see egs_last_hip_error() */
+    EGS_ERR_UNSUPPORTED = -9,
+    EGS_ERR_BAD_STRIDE = -10
+} egs_status;
+
+/* element types; 0..2 are the reference's dtype ids (egs/triton_kernels.py:15-23) */
+typedef enum egs_dtype {
+    EGS_F32 = 0,
+    EGS_F16 = 1,
+    EGS_BF16 = 2,
+    EGS_FP8_E4M3 = 3            /* OCP e4m3fn, weights of the gather only */
+} egs_dtype;
+
+typedef enum egs_index_dtype {
+    EGS_IND_I16 = 0,
+    EGS_IND_I32 = 1,
+    EGS_IND_I64 = 2,
+    EGS_IND_U8 = 3
+} egs_index_dtype;
+
+/* how the weight (or weight gradient) is stored.  The reference passes swapped strides
+ * instead (egs/triton_kernels.py:468, :504, :521). */
+typedef enum egs_w_layout {
+    EGS_W_EIJ = 0,              /* [E, I, J]  gather-side weight  */
+    EGS_W_EJI = 1               /* [E, J, I]  scatter-side weight */
+} egs_w_layout;
+
+typedef enum egs_scatter_mode {
+    EGS_SCATTER_DETERMINISTIC = 0,  /* fixed summation order, bitwise reproducible, no atomics   */
+    EGS_SCATTER_ATOMIC = 1          /* fp32 atomic accumulation, order of additions unspecified  */
+} egs_scatter_mode;
+
+typedef enum egs_op {
+    EGS_OP_GATHER_GEMM = 0,
+    EGS_OP_GEMM_SCATTER = 1,
+    EGS_OP_DW = 2,
+    EGS_OP_GATHER_BACKWARD = 3,     /* GEMM_SCATTER + DW sharing one workspace */
+    EGS_OP_SCATTER_BACKWARD = 4     /* GATHER_GEMM + DW */
+} egs_op;
+
+/* problem sizes shared by every entry point:
+ *   B batches, T tokens per batch, E experts, K picks per (batch, expert),
+ *   I = width of the [B,T,I] side, J = width of the [B,E,K,J] side. */
+typedef struct egs_dims {
+    int32_t B, T, E, K, I, J;
+} egs_dims;
+
+int egs_abi_version(void);
+const char *egs_status_string(int status);
+/* text of the last HIP error seen by the calling thread ("" if none) */
+const char *egs_last_hip_error(void);
+
+/* bytes of scratch the op needs for these sizes (0 is a valid answer).
+ * `mode` is an egs_scatter_mode and only matters for ops that scatter. */
+size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype);
+
+/* ---------------------------------------------------------------------------------------
+ * Kernel-level entry points (one per reference kernel)
+ * ------------------------------------------------------------------------------------- */
+
+/* Y[b,e,k,j] = sum_i X[b, Ind[b,e,k], i] * W(e,i,j)
+ * Replaces expert_gather_kernel (reference egs/triton_kernels.py:49-143).
+ *   X    [B,T,I] act_dtype, strides (ldx_b, ldx_t, 1) in elements
+ *   W    [E,I,J] (EGS_W_EIJ: gather forward) or [E,J,I] (EGS_W_EJI: dY of the scatter), w_dtype
+ *   w_scale  NULL, or for w_dtype == EGS_FP8_E4M3 a float [E,J] per-output-column scale
+ *   Y    [B,E,K,J] act_dtype, dense */
+int egs_gather_gemm(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
+                    const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                    int act_dtype, int w_dtype, int ind_dtype, int w_layout, void *stream);
+
+/* Out[b,t,i] = sum_{e,k : Ind[b,e,k]=t} sum_j Y[b,e,k,j] * W(e,i,j); rows nobody picks are 0.
+ * Replaces expert_scatter_kernel (reference egs/triton_kernels.py:156-247).
+ *   Y    [B,E,K,J] act_dtype, dense
+ *   W    [E,J,I] (EGS_W_EJI: scatter forward) or [E,I,J] (EGS_W_EIJ: dX of the gather), act_dtype
+ *   Out  [B,T,I] act_dtype, dense; fully overwritten */
+int egs_gemm_scatter(const void *Y, const void *W, const void *Ind, void *Out,
+                     void *workspace, size_t workspace_bytes, const egs_dims *d,
+                     int act_dtype, int ind_dtype, int w_layout, int mode, void *stream);
+
+/* dW(e,i,j) = sum_{b,k} Xsrc[b, Ind[b,e,k], i] * Ysrc[b,e,k,j], fp32 accumulation in a fixed
+ * order (split over the batch, then a second fixed-order pass).
+ * Replaces expert_gather_scatter_dW_kernel (reference egs/triton_kernels.py:261-356).
+ *   Xsrc [B,T,I] strides (ldx_b, ldx_t, 1);  Ysrc [B,E,K,J] dense;  both act_dtype
+ *   dW   [E,I,J] (EGS_W_EIJ) or [E,J,I] (EGS_W_EJI) in out_dtype; fully overwritten */
+int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
+           void *workspace, size_t workspace_bytes, const egs_dims *d,
+           int64_t ldx_b, int64_t ldx_t,
+           int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Launcher-level entry points (one per reference callable)
+ * ------------------------------------------------------------------------------------- */
+
+/* expert_gather_forward_call(X, W[E,I,J], Ind) -> Y          reference egs/triton_kernels.py:367-392 */
+int egs_expert_gather_forward(const void *X, const void *W, const void *Ind, void *Y,
+                              const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                              int dtype, int ind_dtype, void *stream);
+
+/* expert_gather_backward_call(X, W[E,I,J], Ind, grad_Y) -> (grad_X, grad_W)   reference :400-441 */
+int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, const void *grad_Y,
+                               void *grad_X, void *grad_W,
+                               void *workspace, size_t workspace_bytes, const egs_dims *d,
+                               int64_t ldx_b, int64_t ldx_t,
+                               int dtype, int ind_dtype, int mode, void *stream);
+
+/* expert_scatter_forward_call(Y, W[E,J,I], Ind, T) -> Out     reference :449-474 */
+int egs_expert_scatter_forward(const void *Y, const void *W, const void *Ind, void *Out,
+                               void *workspace, size_t workspace_bytes, const egs_dims *d,
+                               int dtype, int ind_dtype, int mode, void *stream);
+
+/* expert_scatter_backward_call(Y, W[E,J,I], Ind, grad_Out) -> (grad_Y, grad_W)   reference :483-525 */
+int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, const void *grad_Out,
+                                void *grad_Y, void *grad_W,
+                                void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                int64_t ldg_b, int64_t ldg_t,
+                                int dtype, int ind_dtype, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Debug helper (no counterpart in the reference, which never checks Ind)
+ * ------------------------------------------------------------------------------------- */
+
+/* adds to *d_bad_count (device int32, caller-zeroed) the number of entries outside [0,T) */
+int egs_validate_indices(const void *Ind, int ind_dtype, int64_t n, int32_t T,
+                         int32_t *d_bad_count, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EGS_HIP_H */

@@ -1,0 +1,311 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on the same seeded
+inputs.  Covers the four launchers, both weight layouts, fp32/bf16/fp16, all index widths,
+ragged shapes (the reference draws every dimension from 1..127, test_all.py:97-99),
+duplicate-heavy routing, both scatter modes and the module/autograd surface."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import egs_oracle as O
+from oracle import torch_port as P
+from tests._util import assert_close, make_case, np64
+
+pytestmark = pytest.mark.gpu
+
+import expertscattergather_amd as egs
+from expertscattergather_amd import hip_kernels as hk
+
+hk.create_kernels()
+DEV = "cuda"
+
+# (B, T, E, K, I, J)
+SHAPES = [
+    (2, 16, 3, 8, 32, 16),        # small aligned
+    (4, 64, 8, 16, 128, 64),      # default-like, scaled down
+    (3, 37, 5, 11, 29, 13),       # everything odd, unaligned rows
+    (1, 1, 1, 1, 1, 1),
+    (5, 127, 2, 126, 100, 72),    # tails in every tile dimension
+    (2, 50, 9, 40, 136, 200),     # N > 128: two column tiles; E not a multiple of 8
+    (7, 9, 17, 3, 8, 4),
+    (2, 300, 4, 130, 260, 96),    # several reduction slabs and row tiles
+]
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def dev(t):
+    return t.to(DEV)
+
+
+def run_all(case, T, mode="deterministic"):
+    hk.set_scatter_mode(mode)
+    X, Wg, Ws, Y, dOut, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut", "Ind"))
+    out = {}
+    out["Y"] = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    out["out"] = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    out["dX"], out["dWg"] = hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)
+    out["dY"], out["dWs"] = hk.expert_scatter_backward_call(Y, Ws, Ind, dOut, torch.float32)
+    torch.cuda.synchronize()
+    hk.set_scatter_mode("deterministic")
+    return out
+
+
+def oracle_all(case, T):
+    X, Wg, Ws, Y, dOut = (np64(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut"))
+    Ind = case["Ind"].to(torch.int64).numpy()
+    ref = {}
+    ref["Y"] = O.gather_forward(X, Wg, Ind)
+    ref["out"] = O.scatter_forward(Y, Ws, Ind, T)
+    ref["dX"], ref["dWg"] = O.gather_backward(X, Wg, Ind, Y)
+    ref["dY"], ref["dWs"] = O.scatter_backward(Y, Ws, Ind, dOut)
+    return ref
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_four_launchers_match_oracle(shape, dtype):
+    B, T, E, K, I, J = shape
+    case = make_case(100 + sum(shape), *shape, dtype)
+    got = run_all(case, T)
+    ref = oracle_all(case, T)
+    for name in ("Y", "out", "dX", "dWg", "dY", "dWs"):
+        assert got[name].dtype == dtype
+        assert_close(got[name], ref[name], dtype, f"{name} {shape} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [SHAPES[1], SHAPES[2], SHAPES[5]], ids=lambda s: "x".join(map(str, s)))
+def test_atomic_mode_matches_oracle(shape, dtype):
+    B, T, E, K, I, J = shape
+    case = make_case(7 + sum(shape), *shape, dtype)
+    got = run_all(case, T, mode="atomic")
+    ref = oracle_all(case, T)
+    for name in ("out", "dX"):
+        assert_close(got[name], ref[name], dtype, f"atomic {name} {shape} {dtype}")
+
+
+@pytest.mark.parametrize("ind_dtype", [torch.uint8, torch.int16, torch.int32, torch.int64])
+def test_index_widths_pass_through(ind_dtype):
+    shape = (3, 100, 4, 12, 48, 24)
+    case = make_case(5, *shape, torch.float32, ind_dtype=ind_dtype)
+    before = case["Ind"].clone()
+    got = run_all(case, shape[1])
+    ref = oracle_all(case, shape[1])
+    for name in ("Y", "out", "dX", "dWg", "dY", "dWs"):
+        assert_close(got[name], ref[name], torch.float32, f"{name} {ind_dtype}")
+    assert torch.equal(case["Ind"], before)
+
+
+def test_ind_is_never_written():
+    case = make_case(6, 4, 40, 6, 10, 64, 32, torch.bfloat16)
+    Ind = dev(case["Ind"]); keep = Ind.clone()
+    hk.expert_scatter_forward_call(dev(case["Y"]), dev(case["Ws"]), Ind, 40, torch.float32)
+    hk.expert_gather_backward_call(dev(case["X"]), dev(case["Wg"]), Ind, dev(case["Y"]), torch.float32)
+    torch.cuda.synchronize()
+    assert torch.equal(Ind, keep)
+
+
+def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
+    # all picks of every expert land on 3 tokens: long same-token chains
+    B, T, E, K, I, J = 4, 64, 8, 48, 96, 40
+    case = make_case(9, B, T, E, K, I, J, torch.float32)
+    case["Ind"] = torch.randint(0, 3, (B, E, K), generator=torch.Generator().manual_seed(1))
+    Y, Ws, Ind = dev(case["Y"]), dev(case["Ws"]), dev(case["Ind"])
+    hk.set_scatter_mode("deterministic")
+    first = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    junk = torch.randn(1 << 20, device=DEV)          # disturb the allocator between runs
+    for _ in range(3):
+        again = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+        assert torch.equal(first, again)
+    assert_close(first, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].numpy(), T), torch.float32, "hot tokens")
+    dW1 = hk.expert_gather_backward_call(dev(case["X"]), dev(case["Wg"]), Ind, Y, torch.float32)[1]
+    dW2 = hk.expert_gather_backward_call(dev(case["X"]), dev(case["Wg"]), Ind, Y, torch.float32)[1]
+    assert torch.equal(dW1, dW2)
+    hk.set_scatter_mode("atomic")
+    atomic = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    hk.set_scatter_mode("deterministic")
+    assert_close(atomic, np64(first), torch.float32, "atomic vs deterministic")
+    del junk
+
+
+@pytest.mark.parametrize("mode", ["deterministic", "atomic"])
+def test_scatter_output_does_not_depend_on_stale_memory(mode):
+    # the reference allocates the scatter output with torch.empty and only adds into it
+    # (egs/triton_kernels.py:457); here unpicked tokens must read exactly zero on every call
+    B, T, E, K, I, J = 2, 200, 2, 5, 64, 16
+    case = make_case(11, B, T, E, K, I, J, torch.bfloat16)
+    hk.set_scatter_mode(mode)
+    Y, Ws, Ind = dev(case["Y"]), dev(case["Ws"]), dev(case["Ind"])
+    outs = []
+    for _ in range(3):
+        dirty = torch.full((B, T, I), 7.0, device=DEV, dtype=torch.bfloat16)
+        del dirty                                        # freed block is handed to the next empty()
+        outs.append(hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32).clone())
+    hk.set_scatter_mode("deterministic")
+    picked = torch.zeros(B, T, dtype=torch.bool)
+    picked.scatter_(1, case["Ind"].reshape(B, -1), True)
+    for o in outs:
+        assert (o.cpu()[~picked] == 0).all()
+        assert_close(o, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].numpy(), T), torch.bfloat16, "stale")
+
+
+def test_out_of_range_picks_contribute_nothing():
+    B, T, E, K, I, J = 2, 20, 3, 6, 32, 16
+    case = make_case(13, B, T, E, K, I, J, torch.float32)
+    Ind = case["Ind"].clone()
+    Ind[0, 0, 0] = T; Ind[1, 2, 3] = -1; Ind[1, 1, 1] = 10 ** 9
+    bad = (Ind < 0) | (Ind >= T)
+    assert hk.validate_indices(dev(Ind), T) == int(bad.sum())
+    assert hk.validate_indices(dev(case["Ind"]), T) == 0
+    case2 = dict(case, Ind=Ind)
+    got = run_all(case2, T)
+    # oracle with the bad picks removed: zero their Y rows / route them to a spare token
+    X, Wg, Ws, Y, dOut = (np64(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut"))
+    safe = Ind.clone(); safe[bad] = 0
+    mask = (~bad).numpy()[..., None]
+    refY = O.gather_forward(X, Wg, safe.numpy()) * mask
+    assert_close(got["Y"], refY, torch.float32, "Y with bad picks")
+    assert_close(got["out"], O.scatter_forward(Y * mask, Ws, safe.numpy(), T), torch.float32, "out with bad picks")
+    dX, dWg = O.gather_backward(X, Wg, safe.numpy(), Y * mask)
+    assert_close(got["dX"], dX, torch.float32, "dX with bad picks")
+    assert_close(got["dWg"], dWg, torch.float32, "dWg with bad picks")
+
+
+def test_strided_source_rows():
+    B, T, E, K, I, J = 3, 30, 4, 7, 64, 32
+    case = make_case(17, B, T, E, K, I, J, torch.float32)
+    big = torch.randn(B, T, 2 * I + 8)
+    big[:, :, 8:8 + I] = case["X"]
+    Xs = dev(big)[:, :, 8:8 + I]                      # token stride 2I+8, inner stride 1
+    assert not Xs.is_contiguous()
+    Y = hk.expert_gather_forward_call(Xs, dev(case["Wg"]), dev(case["Ind"]), torch.float32)
+    assert_close(Y, O.gather_forward(np64(case["X"]), np64(case["Wg"]), case["Ind"].numpy()), torch.float32, "strided X")
+    Xt = dev(case["X"].transpose(1, 2).contiguous()).transpose(1, 2)   # inner stride != 1 -> copied
+    Y2 = hk.expert_gather_forward_call(Xt, dev(case["Wg"]), dev(case["Ind"]), torch.float32)
+    assert torch.equal(Y, Y2)
+
+
+def test_empty_inputs():
+    Wg = torch.zeros(3, 8, 4, device=DEV); Ws = torch.zeros(3, 4, 8, device=DEV)
+    X = torch.zeros(2, 5, 8, device=DEV)
+    Ind0 = torch.zeros(2, 3, 0, dtype=torch.int64, device=DEV)
+    assert hk.expert_gather_forward_call(X, Wg, Ind0, torch.float32).shape == (2, 3, 0, 4)
+    out = hk.expert_scatter_forward_call(torch.zeros(2, 3, 0, 4, device=DEV), Ws, Ind0, 5, torch.float32)
+    assert out.shape == (2, 5, 8) and (out == 0).all()
+    dX, dW = hk.expert_gather_backward_call(X, Wg, Ind0, torch.zeros(2, 3, 0, 4, device=DEV), torch.float32)
+    assert (dX == 0).all() and (dW == 0).all()
+
+
+def test_errors_are_python_exceptions():
+    X = torch.zeros(2, 5, 8, device=DEV); W = torch.zeros(3, 8, 4, device=DEV)
+    Ind = torch.zeros(2, 3, 2, dtype=torch.int64, device=DEV)
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        hk.expert_gather_forward_call(X.double(), W.double(), Ind, torch.float32)
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        hk.expert_gather_forward_call(X, W, Ind, torch.int32)
+    with pytest.raises(ValueError):
+        hk.expert_gather_forward_call(X, W.half(), Ind, torch.float32)
+    with pytest.raises(ValueError):
+        hk.expert_gather_forward_call(X, W, Ind.float(), torch.float32)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        hk.expert_gather_forward_call(X.cpu(), W.cpu(), Ind.cpu(), torch.float32)
+
+
+# ------------------------------------------------------------------ module / autograd surface
+@pytest.mark.parametrize("seed", range(5))
+def test_modules_like_the_reference_tests(seed):
+    """Counterpart of the reference's test_all.py: random dims in [1,128), fp32, int16 Ind with
+    replacement, loss = sum, compare forward and both gradients with the torch baseline at
+    atol=1e-3 (test_all.py:9-11)."""
+    g = torch.Generator().manual_seed(seed)
+    B, T, K, E, I, J = torch.randint(1, 128, (6,), generator=g).tolist()
+    torch.manual_seed(seed)
+    X = torch.randn(B, T, I, device=DEV, requires_grad=True)
+    Yin = torch.randn(B, E, K, J, device=DEV, requires_grad=True)
+    Ind = torch.randint(0, T, (B, E, K), generator=g).to(torch.int16).to(DEV)
+    gather = egs.ExpertGather(E, I, J).to(DEV)
+    scatter = egs.ExpertScatter(E, J, I).to(DEV)
+
+    def compare(mine, theirs, name):
+        # the reference's check (test_all.py:9-11): isclose(atol=1e-3), default rtol=1e-5;
+        # the baseline runs in float64 so that only this library's rounding is measured.
+        # W_grad of a sum-loss is a length B*K sum with values in the hundreds, where fp32
+        # accumulation alone costs ~sqrt(B*K)*2^-24 relative: it is held to the fp32 bound
+        # 1e-4 * max|ref| instead of the absolute 1e-3.
+        diff = (mine.detach().cpu().double() - theirs).abs()
+        if name == "W_grad":
+            ok = diff.max().item() <= 1e-4 * theirs.abs().max().item()
+        else:
+            ok = bool((diff <= 1e-3 + 1e-5 * theirs.abs()).all())
+        if not ok:
+            raise AssertionError(f"{name}: max diff {diff.max().item():.3e} dims {(B, T, K, E, I, J)}")
+
+    Y = gather(X, Ind); Y.sum().backward()
+    Xc = X.detach().cpu().double().requires_grad_(True); Wc = gather.W.detach().cpu().double().requires_grad_(True)
+    Yr = P.gather(Xc, Wc, Ind.cpu()); Yr.sum().backward()
+    compare(Y, Yr.detach(), "Y"); compare(X.grad, Xc.grad, "X_grad"); compare(gather.W.grad, Wc.grad, "W_grad")
+
+    out = scatter(Yin, Ind, T); out.sum().backward()
+    Yc = Yin.detach().cpu().double().requires_grad_(True); Wsc = scatter.W.detach().cpu().double().requires_grad_(True)
+    outr = P.scatter(Yc, Wsc, Ind.cpu(), T); outr.sum().backward()
+    compare(out, outr.detach(), "X"); compare(Yin.grad, Yc.grad, "Y_grad"); compare(scatter.W.grad, Wsc.grad, "W_grad")
+
+
+def test_chain_bf16_fwd_bwd_scaled_default_shape():
+    """gather -> scatter -> backward in bf16 through the modules (benchmark step, reduced B)."""
+    from expertscattergather_amd import workloads as wl
+    cfg = wl.CONFIGS["C2"]
+    dims = (8, cfg.T, cfg.E, cfg.K, cfg.I, cfg.J)
+    inp = wl.make_inputs(cfg, dims=dims)
+    B, T, E, K, I, J = dims
+    gather = egs.ExpertGather(E, I, J).to(DEV, torch.bfloat16); scatter = egs.ExpertScatter(E, J, I).to(DEV, torch.bfloat16)
+    with torch.no_grad():
+        gather.W.copy_(inp["Wg"]); scatter.W.copy_(inp["Ws"])
+    X = dev(inp["X"]).requires_grad_(True); Ind = dev(inp["Ind"])
+    Y = gather(X, Ind); out = scatter(Y, Ind, T); out.backward(dev(inp["dOut"]))
+    Xn, Wgn, Wsn, dOn = (np64(inp[k]) for k in ("X", "Wg", "Ws", "dOut")); Indn = inp["Ind"].numpy()
+    Yo = O.gather_forward(Xn, Wgn, Indn)
+    assert_close(Y, Yo, torch.bfloat16, "Y")
+    Yb = np64(Y)                                       # downstream oracles start from the rounded Y
+    assert_close(out, O.scatter_forward(Yb, Wsn, Indn, T), torch.bfloat16, "out")
+    dYo, dWso = O.scatter_backward(Yb, Wsn, Indn, dOn)
+    assert_close(scatter.W.grad, dWso, torch.bfloat16, "dWs")
+    dYb = np64(torch.from_numpy(dYo).to(torch.bfloat16))
+    dXo, dWgo = O.gather_backward(Xn, Wgn, Indn, dYb)
+    assert_close(X.grad, dXo, torch.bfloat16, "dX")
+    assert_close(gather.W.grad, dWgo, torch.bfloat16, "dWg")
+
+
+def test_gather_bias_and_scatter_bias():
+    B, T, E, K, I, J = 2, 12, 3, 5, 16, 8
+    case = make_case(23, B, T, E, K, I, J, torch.float32)
+    gather = egs.ExpertGather(E, I, J, bias=True).to(DEV); scatter = egs.ExpertScatter(E, J, I, bias=True).to(DEV)
+    Ind = dev(case["Ind"])
+    Y = gather(dev(case["X"]), Ind)
+    ref = O.gather_forward(np64(case["X"]), np64(gather.W), case["Ind"].numpy()) + np64(gather.bias)[None]
+    assert_close(Y, ref, torch.float32, "gather bias")
+    out = scatter(dev(case["Y"]), Ind, T)
+    ref = O.scatter_forward(np64(case["Y"]), np64(scatter.W), case["Ind"].numpy(), T)
+    bias = np64(scatter.bias)
+    for b in range(B):
+        for e in range(E):
+            for k in range(K):
+                ref[b, int(case["Ind"][b, e, k])] += bias[e, 0]
+    assert_close(out, ref, torch.float32, "scatter bias")
+
+
+def test_fp8_weight_gather_matches_dequantised_oracle():
+    from expertscattergather_amd import workloads as wl
+    B, T, E, K, I, J = 3, 64, 5, 16, 128, 96
+    case = make_case(29, B, T, E, K, I, J, torch.bfloat16, replace=False)
+    Wq, scale = wl.quantize_fp8_weights(case["Wg"].float())
+    Y = hk.expert_gather_fp8w_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
+    bits = Wq.view(torch.uint8).numpy()
+    ref = O.gather_forward_fp8w(np64(case["X"]), bits, scale.numpy(), case["Ind"].numpy())
+    assert_close(Y, ref, torch.bfloat16, "fp8 weights")
+    # odd sizes take the unaligned byte path
+    B, T, E, K, I, J = 2, 9, 3, 4, 19, 11
+    case = make_case(31, B, T, E, K, I, J, torch.bfloat16)
+    Wq, scale = wl.quantize_fp8_weights(case["Wg"].float())
+    Y = hk.expert_gather_fp8w_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
+    ref = O.gather_forward_fp8w(np64(case["X"]), Wq.view(torch.uint8).numpy(), scale.numpy(), case["Ind"].numpy())
+    assert_close(Y, ref, torch.bfloat16, "fp8 weights odd")
