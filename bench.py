@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused expert gather/scatter path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input at the default shape in
+bf16 (B64 T256 E32 K32 I128 J64): gather forward -> scatter forward -> scatter backward (dY,
+dW_scatter) -> gather backward (dX, dW_gather), i.e. the six kernel-equivalents of a full
+autograd forward+backward.  Inputs are resident in HBM before the timed region starts.
+
+Prints ONE JSON line.  `value` is microseconds per step (lower is better); `roofline`
+describes the dominant kernel (algorithmic bytes / its average launch duration, measured
+with HIP events on the launch stream); `cpu_baseline` is the torch port of the reference's
+baselines timed on the host cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="C2", help="workload (C2 = the metric's configuration)")
+    ap.add_argument("--mode", default=None, choices=["deterministic", "atomic"], help="scatter mode (default: env / deterministic)")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no sharding, no collectives); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from expertscattergather_amd import _abi, hip_kernels as hk, workloads as wl
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    hk.create_kernels()
+    if args.mode:
+        hk.set_scatter_mode(args.mode)
+    cfg = wl.CONFIGS[args.config]
+    B, T, E, K, I, J = cfg.dims
+    inp = wl.make_inputs(cfg)
+    X, Wg, Ws, dOut, Ind = (inp[k].to(dev) for k in ("X", "Wg", "Ws", "dOut", "Ind"))
+    fwd_only = args.config in ("C1", "C5")
+
+    def step():
+        Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+        if fwd_only:
+            return Y, out
+        dY, dWs = hk.expert_scatter_backward_call(Y, Ws, Ind, dOut, torch.float32)
+        dX, dWg = hk.expert_gather_backward_call(X, Wg, Ind, dY, torch.float32)
+        return Y, out, dX, dWg, dWs
+
+    # ------------------------------------------------------------------ whole-step timing
+    for _ in range(max(args.warmup, 3)):
+        step()
+    torch.cuda.synchronize()
+
+    def time_loop(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n
+
+    eager_s = time_loop(step, args.steps)
+    graph_s = None
+    if not args.no_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                for _ in range(3):
+                    step()          # workspace for the capture stream exists before capture
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                keep = step()
+            for _ in range(max(args.warmup, 3)):
+                graph.replay()
+            graph_s = time_loop(graph.replay, args.steps)
+            del keep
+        except Exception as exc:        # report, fall back to the eager number
+            print(f"bench.py: graph capture failed ({exc}); reporting eager timing", file=sys.stderr)
+            graph_s = None
+    step_s = graph_s if graph_s is not None else eager_s
+
+    # ------------------------------------------------------------------ per-kernel timing (HIP events)
+    act = 2 if cfg.dtype != torch.float32 else 4
+    lib = _abi.lib()
+    d = _abi.Dims(B, T, E, K, I, J)
+    dt = hk.dtype_to_type_id(cfg.dtype)
+    stream = torch.cuda.current_stream().cuda_stream
+    Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    out = torch.empty(B, T, I, device=dev, dtype=cfg.dtype)
+    dWbuf = torch.empty(E, I, J, device=dev, dtype=cfg.dtype)
+    mode = 0 if hk.get_scatter_mode() == "deterministic" else 1
+    ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+
+    def k_gather():
+        return lib.egs_gather_gemm(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), None, d, T * I, I, dt, dt, 2, 0, stream)
+
+    def k_scatter():
+        return lib.egs_gemm_scatter(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, d, dt, 2, 1, mode, stream)
+
+    def k_dw():
+        return lib.egs_dw(X.data_ptr(), Y.data_ptr(), Ind.data_ptr(), dWbuf.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, dt, 2, 0, stream)
+
+    def time_kernel(fn, reps):
+        for _ in range(5):
+            assert fn() == 0
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) * 1e-3 / reps
+
+    dims = cfg.dims
+    gemm_bytes = wl.algorithmic_bytes(dims, act)
+    dw_bytes = wl.algorithmic_bytes(dims, act, dw=True)
+    kernels = {
+        "gather_gemm": (time_kernel(k_gather, args.kernel_reps), gemm_bytes),
+        "gemm_scatter": (time_kernel(k_scatter, args.kernel_reps), gemm_bytes),
+        "dw": (time_kernel(k_dw, args.kernel_reps), dw_bytes),
+    }
+    # gather_gemm is the kernel the whole path is named after and runs twice per step
+    dom = "gather_gemm"
+    dom_s, dom_bytes = kernels[dom]
+    n_equiv = 2 if fwd_only else 6
+    chain_bytes = (2 if fwd_only else 4) * gemm_bytes + (0 if fwd_only else 2) * dw_bytes
+    chain_flops = n_equiv * wl.flops(dims)
+
+    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    cpu = None
+    if not args.no_cpu_baseline:
+        from oracle import torch_port as P
+        cores = torch.get_num_threads()
+        Xc, Wgc, Wsc, dOc = (inp[k].float() for k in ("X", "Wg", "Ws", "dOut"))
+        Ic = inp["Ind"]
+
+        def cpu_step():
+            if fwd_only:
+                with torch.no_grad():
+                    return P.scatter(P.gather(Xc, Wgc, Ic), Wsc, Ic, T)
+            return P.chain_fwd_bwd(Xc, Wgc, Wsc, Ic, dOc)
+
+        cpu_step()
+        times = []
+        t_begin = time.perf_counter()
+        while len(times) < 5 and (time.perf_counter() - t_begin < 20.0 or len(times) < 2):
+            t0 = time.perf_counter()
+            cpu_step()
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        cpu = {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us", "cores": cores, "kind": "port",
+               "sample": f"median of {len(times)} full {cfg.name} steps of oracle/torch_port.py (torch CPU, fp32 arithmetic "
+                         f"on the {str(cfg.dtype).split('.')[-1]}-rounded inputs)"}
+
+    result = {
+        "metric": "fused gather+scatter fwd+bwd time per call at B64 T256 E32 K32 I128 J64" if args.config in ("C1", "C2")
+                  else f"fused gather+scatter time per call at {cfg.name}",
+        "value": round(step_s * 1e6, 2),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if cfg.dtype == torch.bfloat16 else str(cfg.dtype).split(".")[-1],
+        "data": "synthetic",
+        "config": {"workload": f"{cfg.name}: B{B} T{T} E{E} K{K} I{I} J{J} {cfg.what}", "scatter_mode": hk.get_scatter_mode(),
+                   "launch": "hip graph replay" if graph_s is not None else "eager"},
+        "step_hbm_gbps": round(chain_bytes / step_s * 1e-9, 1),
+        "step_hbm_frac": round(chain_bytes / step_s * 1e-9 / HBM_PEAK_GBPS, 4),
+        "step_tflops": round(chain_flops / step_s * 1e-12, 2),
+        "eager_us_per_step": round(eager_s * 1e6, 2),
+        "graph_us_per_step": None if graph_s is None else round(graph_s * 1e6, 2),
+        "kernel_us": {k: round(v[0] * 1e6, 2) for k, v in kernels.items()},
+        "kernel_hbm_gbps": {k: round(v[1] / v[0] * 1e-9, 1) for k, v in kernels.items()},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(dom_bytes / dom_s * 1e-9, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_s * 1e6, 3)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
