@@ -61,6 +61,23 @@ __device__ __forceinline__ float f16_bits_to_f32(uint32_t h)
     return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
 }
 
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// two floats -> two 16-bit elements in one dword (round to nearest even; one hardware
+// instruction for bf16 on gfx950)
+template <class TT> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<ElemBF16>(float lo, float hi)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, bf16x2_t));
+}
+template <> __device__ __forceinline__ uint32_t pack2<ElemF16>(float lo, float hi)
+{
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2_t){lo, hi}, f16x2_t));
+}
+template <> __device__ __forceinline__ uint32_t pack2<ElemF32>(float lo, float) { return f32_bits(lo); }
+
 template <class TT> __device__ __forceinline__ uint32_t f32_to_elem_bits(float f);
 template <> __device__ __forceinline__ uint32_t f32_to_elem_bits<ElemF32>(float f) { return f32_bits(f); }
 template <> __device__ __forceinline__ uint32_t f32_to_elem_bits<ElemF16>(float f) { return f32_to_f16_bits(f); }

@@ -11,12 +11,14 @@
 #include "egs_rows_gemm.h"
 #include "egs_dw.h"
 #include "egs_scatter_aux.h"
+#include "egs_small.h"
 
 using namespace egs;
 
 namespace {
 
 thread_local char g_hip_error[256] = "";
+bool g_force_generic = false;      // testing aid: skip the small-expert fast paths
 
 int hip_fail(hipError_t err, const char *what)
 {
@@ -67,22 +69,26 @@ int grid_1d(size_t items, int cap = 8192)
 
 // ------------------------------------------------------------------------------ plans
 struct ScatterPlan {
-    size_t seg_off_at, perm_at, cnt_at, rows_at;   // byte offsets inside the workspace
+    size_t seg_off_at, perm_at, rank_at, cnt_at, rows_at;   // byte offsets inside the workspace
     size_t bytes;
 };
 
+// Workspace of the GEMM-scatter: routing table (segment offsets, picks in token order, scratch
+// ranks, optional global counters) and the product rows in pick order.
+//   deterministic mode: product rows in fp32 -> fp32 accumulation with one final rounding;
+//   atomic ("fast") mode: with 16-bit element types the small-expert kernel keeps the product
+//   rows in the element type (half the traffic, one extra rounding per pick; the summation
+//   order is still fixed); fp32 uses global atomics on the output, no workspace.
+// The rows region is always sized for fp32.
 ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
 {
-    ScatterPlan pl = {0, 0, 0, 0, 0};
+    ScatterPlan pl = {0, 0, 0, 0, 0, 0};
     const size_t N = (size_t)d->E * d->K;
-    if (mode == EGS_SCATTER_ATOMIC) {
-        pl.rows_at = 0;
-        pl.bytes = act_dtype == EGS_F32 ? 0 : align_up((size_t)d->B * d->T * d->I * 4, 256);
-        return pl;
-    }
+    if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) return pl;
     size_t at = 0;
     pl.seg_off_at = at; at += align_up((size_t)d->B * ((size_t)d->T + 1) * 4, 256);
     pl.perm_at = at;    at += align_up((size_t)d->B * N * 4, 256);
+    pl.rank_at = at;    at += align_up((size_t)d->B * N * 4, 256);
     pl.cnt_at = at;     at += d->T > kCsrLdsTokens ? align_up((size_t)d->B * d->T * 4, 256) : 0;
     pl.rows_at = at;    at += align_up((size_t)d->B * N * d->I * 4, 256);
     pl.bytes = at;
@@ -90,13 +96,16 @@ ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
 }
 
 struct DwPlan {
-    int BI, BJ, BK, i_tiles, j_tiles, S, rows_per_split;
-    size_t bytes;
+    int BI, BJ, BK, i_tiles, j_tiles, S, rows_per_split;   // general tiled kernel
+    bool small_ok;                                          // shape admits the small-expert kernel
+    int s_i_tiles, s_j_tiles, s_S, s_rows_per_split;        // its plan
+    size_t bytes;                                           // workspace covering whichever runs
 };
 
 DwPlan plan_dw(const egs_dims *d, int act_dtype)
 {
     DwPlan pl;
+    memset(&pl, 0, sizeof(pl));
     pl.BI = 128; pl.BJ = 64;
     pl.BK = act_dtype == EGS_F32 ? 32 : 64;
     pl.i_tiles = ceil_div(d->I, pl.BI);
@@ -114,6 +123,25 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
     pl.S = (int)S;
     pl.rows_per_split = (int)rows;
     pl.bytes = S > 1 ? align_up((size_t)S * d->E * d->I * d->J * 4, 256) : 0;
+
+    // small experts: 64 x 64 tiles, up to 1024 picks per workgroup, enough workgroups to cover the device
+    pl.small_ok = act_dtype != EGS_F32 && d->I % 8 == 0 && d->J % 8 == 0 && d->I >= 8 && d->J >= 8 && d->I <= 128 &&
+                  d->J <= 128 && Me > 0 && d->E > 0;
+    if (pl.small_ok) {
+        pl.s_i_tiles = ceil_div(d->I, 64);
+        pl.s_j_tiles = ceil_div(d->J, 64);
+        const int64_t tiles = (int64_t)d->E * pl.s_i_tiles * pl.s_j_tiles;
+        int64_t s2 = (256 + tiles - 1) / tiles;
+        const int64_t need = (Me + kDwSmallMaxRows - 1) / kDwSmallMaxRows, most = (Me + 127) / 128;
+        if (s2 < need) s2 = need;
+        if (s2 > most) s2 = most;
+        int64_t r2 = ((Me + s2 - 1) / s2 + 127) / 128 * 128;
+        s2 = (Me + r2 - 1) / r2;
+        pl.s_S = (int)s2;
+        pl.s_rows_per_split = (int)r2;
+        const size_t b2 = s2 > 1 ? align_up((size_t)s2 * d->E * d->I * d->J * 4, 256) : 0;
+        if (b2 > pl.bytes) pl.bytes = b2;
+    }
     return pl;
 }
 
@@ -162,12 +190,161 @@ int launch_rows_gemm(RowsGemmParams &p, int act_dtype, bool w_trans, hipStream_t
     }
 }
 
+// ------------------------------------------------------------------------------ small-expert fast paths
+size_t device_lds_limit()
+{
+    static size_t limit = 0;
+    if (limit == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0)
+            limit = (size_t)v;
+        else
+            limit = 64 * 1024;
+    }
+    return limit;
+}
+
+constexpr uint64_t kSpan32 = 0xFFFFFFFFull;      // the small kernel addresses with 32-bit byte offsets
+
+template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
+int launch_rows_small_ks(SmallRowsParams &p, int R, size_t lds, hipStream_t s)
+{
+    const int grid = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
+    switch (R) {
+    case 32: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
+    case 64: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
+    default: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 4, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
+    }
+    EGS_CHECK_LAUNCH("rows_small_kernel");
+    return EGS_OK;
+}
+
+template <class TT, bool GATHER, bool OUT_F32>
+int launch_rows_small(SmallRowsParams &p, int R, bool nmajor, size_t lds, hipStream_t s)
+{
+    if (p.N <= 64)
+        return nmajor ? launch_rows_small_ks<TT, true, 4, GATHER, OUT_F32>(p, R, lds, s)
+                      : launch_rows_small_ks<TT, false, 4, GATHER, OUT_F32>(p, R, lds, s);
+    return nmajor ? launch_rows_small_ks<TT, true, 8, GATHER, OUT_F32>(p, R, lds, s)
+                  : launch_rows_small_ks<TT, false, 8, GATHER, OUT_F32>(p, R, lds, s);
+}
+
+bool small_shape_ok(int act_dtype, int R, int N)
+{
+    return act_dtype != EGS_F32 && (R == 32 || R == 64 || R == 128) && N % 8 == 0 && N >= 8 && N <= 128;
+}
+
+// Both return 1 if the problem does not qualify (caller takes the general kernel), else a status.
+int try_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
+                     int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, hipStream_t s)
+{
+    const int R = d->I, N = d->J;
+    if (w_dtype != act_dtype || !small_shape_ok(act_dtype, R, N)) return 1;
+    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16)) return 1;
+    if ((ldx_b * 2) % 16 || (ldx_t * 2) % 16 || d->T == 0) return 1;
+    const int64_t Me = (int64_t)d->B * d->K;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + R) * 2;
+    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32 || (uint64_t)Me * d->E * N * 2 > kSpan32) return 1;
+    SmallRowsParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
+    p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
+    p.tiles_per_e = (int)((Me + 255) / 256);
+    if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e > INT32_MAX) return 1;
+    const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
+    return act_dtype == EGS_BF16 ? launch_rows_small<ElemBF16, true, false>(p, R, nmajor, 0, s)
+                                 : launch_rows_small<ElemF16, true, false>(p, R, nmajor, 0, s);
+}
+
+// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
+size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
+
+// product rows of the scatter in pick order; when `csr` is set the routing table is built by
+// extra workgroups of the same launch
+int try_scatter_rows_small(const void *Y, const void *W, void *rows, bool rows_f32, const egs_dims *d, int act_dtype,
+                           int w_layout, bool csr, const void *Ind, int ind_dtype, int32_t *seg_off, int32_t *perm,
+                           int32_t *rank_tmp, hipStream_t s)
+{
+    const int R = d->J, N = d->I;
+    if (!small_shape_ok(act_dtype, R, N)) return 1;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16)) return 1;
+    const int64_t Me = (int64_t)d->B * d->K;
+    if ((uint64_t)Me * d->E * R * 2 > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32 ||
+        (uint64_t)Me * d->E * N * 4 > kSpan32) return 1;
+    SmallRowsParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)Y; p.W = (const char *)W; p.C = (char *)rows;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
+    p.tiles_per_e = (int)((Me + 255) / 256);
+    size_t lds = 0;
+    if (csr) {
+        p.csr_blocks = d->B; p.Ind = Ind; p.ind_dtype = ind_dtype;
+        p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp;
+        lds = csr_count_lds(d->T, 4);
+    }
+    if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e + p.csr_blocks > INT32_MAX) return 1;
+    const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
+    if (act_dtype == EGS_BF16)
+        return rows_f32 ? launch_rows_small<ElemBF16, false, true>(p, R, nmajor, lds, s)
+                        : launch_rows_small<ElemBF16, false, false>(p, R, nmajor, lds, s);
+    return rows_f32 ? launch_rows_small<ElemF16, false, true>(p, R, nmajor, lds, s)
+                    : launch_rows_small<ElemF16, false, false>(p, R, nmajor, lds, s);
+}
+
+// routing table of the deterministic scatter as a launch of its own: counting sort with
+// per-wavefront histograms when they fit in LDS, bitonic sort in LDS for long sequences, else
+// the one-wavefront counting sort
+int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int32_t *seg_off, int32_t *perm,
+                         int32_t *rank_tmp, int32_t *cnt, hipStream_t s)
+{
+    const int64_t N = (int64_t)d->E * d->K;
+    if (N >= 1) {
+        int nw = (int)((N + 63) / 64);
+        if (nw > 16) nw = 16;
+        while (nw > 1 && csr_count_lds(d->T, nw) > 64 * 1024) nw >>= 1;
+        const size_t lds = csr_count_lds(d->T, nw);
+        if (lds <= 64 * 1024 && (nw > 1 || N <= 4096)) {
+            hipLaunchKernelGGL(csr_count_kernel, dim3(d->B), dim3(64 * nw), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, rank_tmp);
+            EGS_CHECK_LAUNCH("csr_count_kernel");
+            return EGS_OK;
+        }
+    }
+    int NP = 1, QB = 0;
+    while (NP < N) { NP <<= 1; ++QB; }
+    const bool sortable = N >= 1 && NP <= 32768 && (((uint64_t)d->T << QB) <= 0xFFFFFFFFull);
+    if (sortable) {
+        const size_t lds = (size_t)NP * 4;
+        static size_t configured = 64 * 1024;
+        if (lds > configured) {
+            hipError_t err = hipFuncSetAttribute((const void *)csr_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(csr_sort_kernel)");
+            configured = lds;
+        }
+        int threads = NP / 2;
+        if (threads < 64) threads = 64;
+        if (threads > 1024) threads = 1024;
+        hipLaunchKernelGGL(csr_sort_kernel, dim3(d->B), dim3(threads), lds, s, Ind, ind_dtype, d->T, (int32_t)N, NP, QB, seg_off, perm);
+        EGS_CHECK_LAUNCH("csr_sort_kernel");
+        return EGS_OK;
+    }
+    const size_t lds = d->T > kCsrLdsTokens ? 0 : (size_t)d->T * 4;
+    hipLaunchKernelGGL(csr_build_kernel, dim3(d->B), dim3(kWave), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, cnt);
+    EGS_CHECK_LAUNCH("csr_build_kernel");
+    return EGS_OK;
+}
+
 // ------------------------------------------------------------------------------ implementations
 int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
                      const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
                      int w_layout, hipStream_t s)
 {
     const int ES = elem_size(act_dtype), WES = elem_size(w_dtype);
+    if (w_scale == nullptr && !g_force_generic) {
+        int rc = try_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, s);
+        if (rc != 1) return rc;
+    }
     RowsGemmParams p;
     memset(&p, 0, sizeof(p));
     p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y; p.w_scale = w_scale;
@@ -208,53 +385,64 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     const int64_t w_row = w_trans ? d->I : d->J;
     p.w_vec = aligned_to(W, 16) && (w_row * ES) % 16 == 0;
 
-    if (mode == EGS_SCATTER_ATOMIC) {
-        float *acc32 = act_dtype == EGS_F32 ? (float *)Out : (float *)(ws + pl.rows_at);
+    if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) {
+        float *acc32 = (float *)Out;
         hipLaunchKernelGGL(fill_zero_f32_kernel, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s, acc32, out_elems,
                            (int)aligned_to(acc32, 16));
         EGS_CHECK_LAUNCH("fill_zero_f32_kernel");
         p.C = (char *)acc32;
         p.c_vec = 0;
-        int rc = launch_rows_gemm<false, EPI_ATOMIC_F32>(p, act_dtype, w_trans, s);
-        if (rc != EGS_OK) return rc;
-        if (act_dtype != EGS_F32) {
-            const int vec = (int)aligned_to(Out, 8);
-            if (act_dtype == EGS_BF16)
-                hipLaunchKernelGGL(downconvert_kernel<ElemBF16>, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s,
-                                   (const float *)acc32, (uint16_t *)Out, out_elems, vec);
-            else
-                hipLaunchKernelGGL(downconvert_kernel<ElemF16>, dim3(grid_1d(out_elems / 4 + 1)), dim3(kThreads), 0, s,
-                                   (const float *)acc32, (uint16_t *)Out, out_elems, vec);
-            EGS_CHECK_LAUNCH("downconvert_kernel");
-        }
-        return EGS_OK;
+        return launch_rows_gemm<false, EPI_ATOMIC_F32>(p, act_dtype, w_trans, s);
     }
 
-    // deterministic: routing table, fp32 product rows, fixed-order reduction per token
+    // routing table (picks in token order) + product rows in pick order, then one fixed-order
+    // gather-and-sum per token that writes every output row exactly once
     int32_t *seg_off = (int32_t *)(ws + pl.seg_off_at);
     int32_t *perm = (int32_t *)(ws + pl.perm_at);
+    int32_t *rank_tmp = (int32_t *)(ws + pl.rank_at);
     int32_t *cnt = d->T > kCsrLdsTokens ? (int32_t *)(ws + pl.cnt_at) : nullptr;
-    float *rows = (float *)(ws + pl.rows_at);
-    const size_t lds = d->T > kCsrLdsTokens ? 0 : (size_t)d->T * 4;
-    hipLaunchKernelGGL(csr_build_kernel, dim3(d->B), dim3(kWave), lds, s, Ind, ind_dtype, d->T, N, seg_off, perm, cnt);
-    EGS_CHECK_LAUNCH("csr_build_kernel");
-    p.C = (char *)rows;
-    p.c_vec = d->I % 4 == 0;
-    int rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
+    void *rows = ws + pl.rows_at;
+    bool rows_f32 = (mode == EGS_SCATTER_DETERMINISTIC);
+    int rc = 1;
+    if (!g_force_generic && N > 0) {
+        // small experts: the sort rides along with the product when its histograms are small
+        const bool ride = csr_count_lds(d->T, 4) <= 16 * 1024 && N <= 4096;
+        if (!ride) {
+            rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
+            if (rc != EGS_OK) return rc;
+        }
+        rc = try_scatter_rows_small(Y, W, rows, rows_f32, d, act_dtype, w_layout, ride, Ind, ind_dtype, seg_off, perm,
+                                    rank_tmp, s);
+        if (rc == 1 && ride) {
+            rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
+            if (rc != EGS_OK) return rc;
+            rc = 1;
+        }
+    } else {
+        rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
+        if (rc != EGS_OK) return rc;
+        rc = 1;
+    }
+    if (rc == 1) {
+        rows_f32 = true;                    // the general kernel writes fp32 rows
+        p.C = (char *)rows;
+        p.c_vec = d->I % 4 == 0;
+        rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
+    }
     if (rc != EGS_OK) return rc;
     const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
     const size_t items = (size_t)d->B * d->T * (vw4 ? d->I / 4 : d->I);
     const int grid = grid_1d(items, 65536);
-#define EGS_SEGSUM(TT)                                                                                              \
+#define EGS_SEGSUM(TT, PT)                                                                                          \
     do {                                                                                                            \
-        if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, 4>), dim3(grid), dim3(kThreads), 0, s, rows, seg_off,   \
-                                    perm, (char *)Out, d->B, d->T, N, d->I);                                        \
-        else hipLaunchKernelGGL((segment_sum_kernel<TT, 1>), dim3(grid), dim3(kThreads), 0, s, rows, seg_off, perm, \
-                                (char *)Out, d->B, d->T, N, d->I);                                                  \
+        if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 4>), dim3(grid), dim3(kThreads), 0, s,              \
+                                    (const PT *)rows, seg_off, perm, (char *)Out, d->B, d->T, N, d->I);             \
+        else hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 1>), dim3(grid), dim3(kThreads), 0, s,                  \
+                                (const PT *)rows, seg_off, perm, (char *)Out, d->B, d->T, N, d->I);                 \
     } while (0)
-    if (act_dtype == EGS_F32) EGS_SEGSUM(ElemF32);
-    else if (act_dtype == EGS_F16) EGS_SEGSUM(ElemF16);
-    else EGS_SEGSUM(ElemBF16);
+    if (act_dtype == EGS_F32) EGS_SEGSUM(ElemF32, float);
+    else if (act_dtype == EGS_F16) { if (rows_f32) EGS_SEGSUM(ElemF16, float); else EGS_SEGSUM(ElemF16, uint16_t); }
+    else { if (rows_f32) EGS_SEGSUM(ElemBF16, float); else EGS_SEGSUM(ElemBF16, uint16_t); }
 #undef EGS_SEGSUM
     EGS_CHECK_LAUNCH("segment_sum_kernel");
     return EGS_OK;
@@ -267,6 +455,36 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
     if (w_elems == 0) return EGS_OK;
     const int ES = elem_size(act_dtype), OES = elem_size(out_dtype);
     const DwPlan pl = plan_dw(d, act_dtype);
+    if (pl.small_ok && !g_force_generic) {
+        const uint64_t x_span = d->T > 0 ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * 2 : 0;
+        const bool ok = d->T > 0 && aligned_to(Xs, 16) && aligned_to(Ys, 16) && aligned_to(dW, 16) && (ldx_b * 2) % 16 == 0 &&
+                        (ldx_t * 2) % 16 == 0 && x_span <= kSpan32 &&
+                        (uint64_t)d->B * d->E * d->K * d->J * 2 <= kSpan32 &&
+                        (int64_t)8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S <= INT32_MAX;
+        if (ok) {
+            SmallDwParams q;
+            memset(&q, 0, sizeof(q));
+            q.Xs = (const char *)Xs; q.Ys = (const char *)Ys; q.Ind = Ind; q.part = (float *)workspace; q.dW = (char *)dW;
+            q.B = d->B; q.T = d->T; q.E = d->E; q.K = d->K; q.I = d->I; q.J = d->J;
+            q.ldx_b = ldx_b; q.ldx_t = ldx_t; q.ind_dtype = ind_dtype;
+            q.i_tiles = pl.s_i_tiles; q.j_tiles = pl.s_j_tiles; q.S = pl.s_S; q.rows_per_split = pl.s_rows_per_split;
+            q.out_dtype = out_dtype; q.dw_layout = dw_layout;
+            const int grid = 8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S;
+            if (act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_small_kernel<ElemBF16>, dim3(grid), dim3(kThreads), 0, s, q);
+            else hipLaunchKernelGGL(dw_small_kernel<ElemF16>, dim3(grid), dim3(kThreads), 0, s, q);
+            EGS_CHECK_LAUNCH("dw_small_kernel");
+            if (pl.s_S > 1) {
+                if (dw_layout == EGS_W_EIJ && w_elems % 4 == 0)
+                    hipLaunchKernelGGL(dw_reduce4_kernel, dim3(grid_1d(w_elems / 4, 2048)), dim3(kThreads), 0, s,
+                                       (const float *)workspace, (char *)dW, pl.s_S, w_elems / 4, out_dtype);
+                else
+                    hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s,
+                                       (const float *)workspace, (char *)dW, pl.s_S, d->E, d->I, d->J, out_dtype, dw_layout);
+                EGS_CHECK_LAUNCH("dw_reduce_kernel");
+            }
+            return EGS_OK;
+        }
+    }
     DwParams p;
     memset(&p, 0, sizeof(p));
     p.Xs = (const char *)Xs; p.Ys = (const char *)Ys; p.Ind = Ind;
@@ -392,6 +610,8 @@ const char *egs_status_string(int status)
 }
 
 const char *egs_last_hip_error(void) { return g_hip_error; }
+
+void egs_set_force_generic(int on) { g_force_generic = on != 0; }
 
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
 {

@@ -237,8 +237,8 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
                         *reinterpret_cast<f32x4 *>(crow + (size_t)n * 4) = v;
                     } else {
                         u32x2 w;
-                        w[0] = f32_to_elem_bits<TT>(v[0]) | (f32_to_elem_bits<TT>(v[1]) << 16);
-                        w[1] = f32_to_elem_bits<TT>(v[2]) | (f32_to_elem_bits<TT>(v[3]) << 16);
+                        w[0] = pack2<TT>(v[0], v[1]);
+                        w[1] = pack2<TT>(v[2], v[3]);
                         *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = w;
                     }
                 } else {

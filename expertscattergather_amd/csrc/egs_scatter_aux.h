@@ -23,12 +23,15 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane)
     return v;
 }
 
-// One wavefront per batch builds, for its [E*K] picks, a stable counting sort by token:
-//   seg_off[b][t] .. seg_off[b][t+1]  = positions in perm[b] of the picks that selected t
-//   perm[b][pos]                      = pick number q = e*K + k, increasing inside a segment
-// Stability (picks of one token stay in increasing q) is what fixes the summation order of
-// the deterministic scatter.  Ranks inside a 64-pick chunk come from ballots over the bits of
-// the token id, not from atomics, so the result does not depend on hardware ordering.
+// Routing table of one batch element: its [N = E*K] picks in a stable order by token,
+//   seg_off[b][t] .. seg_off[b][t+1]  = sorted positions of the picks that selected token t
+//   perm[b][s]                        = pick q = e*K + k at sorted position s, increasing inside
+//                                       a token's segment (picks with a bad index are left out)
+// Stability is what fixes the summation order of the deterministic scatter.
+//
+// General version: one wavefront per batch element does a counting sort.  Ranks inside a
+// 64-pick chunk come from ballots over the bits of the token id, not from atomics, so the
+// result does not depend on hardware ordering.  Works for any T and N; slow for large N.
 __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
                                                           int32_t *seg_off, int32_t *perm, int32_t *cnt_global)
 {
@@ -82,12 +85,144 @@ __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32
     }
 }
 
-// out[b,t,:] = sum over the picks of token t, in perm order, of the fp32 rows P[b, pick, :];
-// every row of out is written exactly once (tokens nobody picked become zero).
-template <class TT, int VW>
-__global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float *P, const int32_t *seg_off,
-                                                               const int32_t *perm, char *out, int32_t B, int32_t T,
-                                                               int32_t N, int32_t I)
+// Fast version when T counters per wavefront fit in LDS: one workgroup of NW wavefronts per
+// batch element.  Wavefront w ranks the picks of its contiguous slice against a private
+// histogram (ballot matching inside each 64-pick chunk, no atomics), then the per-token counts
+// are prefix-summed over wavefronts and over tokens, and every pick goes to
+//   start of its token + picks of that token in earlier slices + rank inside its slice.
+// LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch.
+__device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, int nthreads, const void *Ind,
+                                               int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
+                                               int32_t *perm, int32_t *rank_tmp)
+{
+    const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
+    int32_t *hist = sh_cnt + (size_t)wave * T;          // this wavefront's counters
+    int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
+    const int64_t base_pick = (int64_t)b * N;
+    const int slice = ((N + NW - 1) / NW + 63) & ~63;
+    const int q_begin = wave * slice, q_end = min(N, q_begin + slice);
+
+    for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
+    __syncthreads();
+
+    const int nbits = T > 1 ? 32 - __clz(T - 1) : 0;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
+        const int q = q0 + lane;
+        const int32_t t = q < q_end ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+        uint64_t same = __ballot(t >= 0);
+        for (int bit = 0; bit < nbits; ++bit) {
+            const bool one = (t >> bit) & 1;
+            const uint64_t bal = __ballot(one);
+            same &= one ? bal : ~bal;
+        }
+        if (t >= 0) {
+            const int rank = __popcll(same & lt_mask), group = __popcll(same);
+            const int start = cnt_load(&hist[t]);
+            rank_tmp[base_pick + q] = start + rank;         // rank inside this slice
+            if (rank == group - 1) cnt_store(&hist[t], start + group);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+
+    // per token: counts -> exclusive prefix over wavefronts; total per token
+    for (int t = tid; t < T; t += nthreads) {
+        int run = 0;
+        for (int w = 0; w < NW; ++w) {
+            const int c = sh_cnt[(size_t)w * T + t];
+            sh_cnt[(size_t)w * T + t] = run;
+            run += c;
+        }
+        tok_start[t] = run;
+    }
+    __syncthreads();
+    if (wave == 0) {                                        // exclusive scan of the totals over tokens
+        int running = 0;
+        for (int t0 = 0; t0 < T; t0 += kWave) {
+            const int t = t0 + lane;
+            const int c = t < T ? tok_start[t] : 0;
+            const int incl = wave_inclusive_scan(c, lane);
+            if (t < T) tok_start[t] = running + incl - c;
+            running += __shfl(incl, kWave - 1, kWave);
+        }
+        if (lane == 0) tok_start[T] = running;
+    }
+    __syncthreads();
+    for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)b * (T + 1) + t] = tok_start[t];
+    for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
+        const int q = q0 + lane;
+        if (q < q_end) {
+            const int32_t t = load_token(Ind, ind_dtype, base_pick + q, T);
+            if (t >= 0) perm[base_pick + tok_start[t] + hist[t] + rank_tmp[base_pick + q]] = q;
+        }
+    }
+}
+
+__global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
+                                                         int32_t *seg_off, int32_t *perm, int32_t *rank_tmp)
+{
+    extern __shared__ int32_t sh_cnt_dyn[];
+    csr_count_body(sh_cnt_dyn, (int)blockIdx.x, (int)threadIdx.x, (int)blockDim.x, Ind, ind_dtype, T, N, seg_off, perm,
+                   rank_tmp);
+}
+
+// Fast version for N <= 32768 picks whose (token, pick) pair fits 32 bits: one workgroup per
+// batch element sorts the keys (token << QB | q) with a bitonic network in LDS.  Keys are
+// unique, so the sorted order is the stable order by token.  NP = N rounded up to a power of
+// two; dynamic LDS = NP * 4 bytes.
+__global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
+                                                        int32_t NP, int32_t QB, int32_t *seg_off, int32_t *perm)
+{
+    extern __shared__ uint32_t keys[];
+    const int tid = (int)threadIdx.x, nthreads = (int)blockDim.x, b = (int)blockIdx.x;
+    const int64_t base_pick = (int64_t)b * N;
+    for (int q = tid; q < NP; q += nthreads) {
+        uint32_t key = 0xFFFFFFFFu;
+        if (q < N) {
+            int32_t t = load_token(Ind, ind_dtype, base_pick + q, T);
+            if (t >= 0) key = ((uint32_t)t << QB) | (uint32_t)q;
+        }
+        keys[q] = key;
+    }
+    __syncthreads();
+    for (int k = 2; k <= NP; k <<= 1) {
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int i = tid; i < (NP >> 1); i += nthreads) {
+                // pair (lo, lo + j) of the j-stride butterfly
+                const int lo = ((i & ~(j - 1)) << 1) | (i & (j - 1));
+                const int hi = lo + j;
+                const bool ascending = (lo & k) == 0;
+                const uint32_t x = keys[lo], y = keys[hi];
+                if ((x > y) == ascending) { keys[lo] = y; keys[hi] = x; }
+            }
+            __syncthreads();
+        }
+    }
+    const uint32_t qmask = (1u << QB) - 1u;
+    for (int s = tid; s < N; s += nthreads) {
+        const uint32_t key = keys[s];
+        if (key != 0xFFFFFFFFu) perm[base_pick + s] = (int32_t)(key & qmask);
+    }
+    // seg_off[t] = number of keys below (t << QB); seg_off[T] = number of valid keys
+    for (int t = tid; t <= T; t += nthreads) {
+        const uint32_t want = t < T ? ((uint32_t)t << QB) : 0xFFFFFFFFu;
+        int lo = 0, hi = NP;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (keys[mid] < want) lo = mid + 1; else hi = mid;
+        }
+        seg_off[(size_t)b * (T + 1) + t] = lo;
+    }
+}
+
+// out[b,t,:] = sum, in routing-table order, of the product rows of the picks of token t
+// (rows perm[b][s] of P[b], seg_off[t] <= s < seg_off[t+1]); every row of out is written
+// exactly once (tokens nobody picked become zero).  P rows hold PT (float, or 16-bit values
+// of the element type TT); VW elements per thread.
+template <class TT, class PT, int VW>
+__global__ __launch_bounds__(kThreads) void segment_sum_kernel(const PT *P, const int32_t *seg_off, const int32_t *perm,
+                                                               char *out, int32_t B, int32_t T, int32_t N, int32_t I)
 {
     const int IV = (I + VW - 1) / VW;
     const size_t items = (size_t)B * T * IV;
@@ -101,14 +236,28 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float *P, c
 #pragma unroll
         for (int x = 0; x < VW; ++x) acc[x] = 0.f;
         for (int s = s0; s < s1; ++s) {
-            int q = perm[(size_t)b * N + s];
-            const float *src = P + ((size_t)b * N + q) * I + (size_t)iv * VW;
-            if constexpr (VW == 4) {
-                f32x4 v = *reinterpret_cast<const f32x4 *>(src);
+            const int q = perm[(size_t)b * N + s];
+            const PT *src = P + ((size_t)b * N + q) * I + (size_t)iv * VW;
+            if constexpr (sizeof(PT) == 4) {
+                if constexpr (VW == 4) {
+                    f32x4 v = *reinterpret_cast<const f32x4 *>(src);
 #pragma unroll
-                for (int x = 0; x < 4; ++x) acc[x] += v[x];
+                    for (int x = 0; x < 4; ++x) acc[x] += v[x];
+                } else {
+                    acc[0] += src[0];
+                }
             } else {
-                acc[0] += src[0];
+                if constexpr (VW == 4) {
+                    u32x2 v = *reinterpret_cast<const u32x2 *>(src);
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        uint32_t hbits = (v[x >> 1] >> (16 * (x & 1))) & 0xffffu;
+                        acc[x] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
+                    }
+                } else {
+                    uint32_t hbits = (uint32_t)src[0];
+                    acc[0] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
+                }
             }
         }
         size_t at = row * I + (size_t)iv * VW;
@@ -120,8 +269,8 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const float *P, c
             uint16_t *dst = reinterpret_cast<uint16_t *>(out) + at;
             if constexpr (VW == 4) {
                 u32x2 w;
-                w[0] = f32_to_elem_bits<TT>(acc[0]) | (f32_to_elem_bits<TT>(acc[1]) << 16);
-                w[1] = f32_to_elem_bits<TT>(acc[2]) | (f32_to_elem_bits<TT>(acc[3]) << 16);
+                w[0] = pack2<TT>(acc[0], acc[1]);
+                w[1] = pack2<TT>(acc[2], acc[3]);
                 *reinterpret_cast<u32x2 *>(dst) = w;
             } else {
                 dst[0] = (uint16_t)f32_to_elem_bits<TT>(acc[0]);
@@ -151,8 +300,8 @@ __global__ __launch_bounds__(kThreads) void downconvert_kernel(const float *src,
     for (size_t i = gid; i < n4; i += stride) {
         f32x4 v = reinterpret_cast<const f32x4 *>(src)[i];
         u32x2 w;
-        w[0] = f32_to_elem_bits<TT>(v[0]) | (f32_to_elem_bits<TT>(v[1]) << 16);
-        w[1] = f32_to_elem_bits<TT>(v[2]) | (f32_to_elem_bits<TT>(v[3]) << 16);
+        w[0] = pack2<TT>(v[0], v[1]);
+        w[1] = pack2<TT>(v[2], v[3]);
         reinterpret_cast<u32x2 *>(dst)[i] = w;
     }
     for (size_t i = n4 * 4 + gid; i < n; i += stride) dst[i] = (uint16_t)f32_to_elem_bits<TT>(src[i]);

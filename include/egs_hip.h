@@ -92,6 +92,10 @@ const char *egs_status_string(int status);
 /* text of the last HIP error seen by the calling thread ("" if none) */
 const char *egs_last_hip_error(void);
 
+/* Testing aid: non-zero routes every call through the general tiled kernels, skipping the
+ * specialised small-expert kernels (both must give results within the same tolerances). */
+void egs_set_force_generic(int on);
+
 /* bytes of scratch the op needs for these sizes (0 is a valid answer).
  * `mode` is an egs_scatter_mode and only matters for ops that scatter. */
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype);

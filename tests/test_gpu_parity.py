@@ -60,9 +60,30 @@ def oracle_all(case, T):
     return ref
 
 
+# shapes that qualify for the small-expert kernels (16-bit, reduction length 32/64/128, output
+# width a multiple of 8 and <= 64 for the gather, K <= 64 for the scatter), with ragged K, T, E
+SMALL_SHAPES = [
+    (3, 50, 9, 11, 64, 32),       # ragged K, T, E; expert groups of unequal size
+    (2, 33, 5, 64, 128, 64),      # K = 64: four row tiles, E < 8: one expert group
+    (5, 20, 3, 7, 32, 8),
+    (2, 256, 32, 32, 128, 64),    # two batch elements of the default shape
+    (9, 40, 12, 33, 128, 32),     # K = 33
+    (2, 700, 8, 20, 32, 64),      # long T: accumulators of one expert group fill the LDS
+    (3, 64, 16, 16, 64, 56),      # J not a multiple of 16 (gather columns), scatter takes the general path
+]
+
+
+@pytest.fixture(params=[False, True], ids=["fastpaths", "generic"])
+def force_generic(request):
+    from expertscattergather_amd import _abi
+    _abi.lib().egs_set_force_generic(1 if request.param else 0)
+    yield request.param
+    _abi.lib().egs_set_force_generic(0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])
-@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
-def test_four_launchers_match_oracle(shape, dtype):
+@pytest.mark.parametrize("shape", SHAPES + SMALL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_four_launchers_match_oracle(shape, dtype, force_generic):
     B, T, E, K, I, J = shape
     case = make_case(100 + sum(shape), *shape, dtype)
     got = run_all(case, T)
