@@ -18,7 +18,8 @@ using namespace egs;
 namespace {
 
 thread_local char g_hip_error[256] = "";
-bool g_force_generic = false;      // testing aid: skip the small-expert fast paths
+bool g_force_generic = false;
+unsigned long long *g_dbg_times = nullptr;   // performance debugging: per-wavefront time stamps of the small rows kernel      // testing aid: skip the small-expert fast paths
 
 int hip_fail(hipError_t err, const char *what)
 {
@@ -211,6 +212,7 @@ template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
 int launch_rows_small_ks(SmallRowsParams &p, int R, size_t lds, hipStream_t s)
 {
     const int grid = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
+    p.dbg_times = g_dbg_times;
     switch (R) {
     case 32: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
     case 64: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
@@ -612,6 +614,7 @@ const char *egs_status_string(int status)
 const char *egs_last_hip_error(void) { return g_hip_error; }
 
 void egs_set_force_generic(int on) { g_force_generic = on != 0; }
+void egs_set_debug_times(void *buf) { g_dbg_times = (unsigned long long *)buf; }
 
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
 {

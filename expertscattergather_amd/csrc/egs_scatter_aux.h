@@ -3,6 +3,7 @@
 // the zero-fill / down-convert passes of the atomic mode.
 #pragma once
 #include "egs_device.h"
+#include <type_traits>
 
 namespace egs {
 
@@ -95,34 +96,57 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
                                                int32_t *perm, int32_t *rank_tmp)
 {
+    constexpr int MAXC = 4;                             // 64-pick chunks whose tokens and ranks stay in registers
     const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
     int32_t *hist = sh_cnt + (size_t)wave * T;          // this wavefront's counters
     int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
     const int64_t base_pick = (int64_t)b * N;
     const int slice = ((N + NW - 1) / NW + 63) & ~63;
     const int q_begin = wave * slice, q_end = min(N, q_begin + slice);
+    const bool in_regs = slice <= MAXC * kWave;
+
+    // tokens of the slice go in flight before anything else
+    int32_t tk[MAXC], rk[MAXC];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int q = q_begin + c * kWave + lane;
+        tk[c] = (in_regs && q < q_end) ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+        rk[c] = 0;
+    }
 
     for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
     __syncthreads();
 
     const int nbits = T > 1 ? 32 - __clz(T - 1) : 0;
     const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
-        const int q = q0 + lane;
-        const int32_t t = q < q_end ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+    auto rank_chunk = [&](int32_t t) -> int {           // rank of this lane's pick among equal tokens seen so far by this wavefront
         uint64_t same = __ballot(t >= 0);
         for (int bit = 0; bit < nbits; ++bit) {
             const bool one = (t >> bit) & 1;
             const uint64_t bal = __ballot(one);
             same &= one ? bal : ~bal;
         }
+        int r = 0;
         if (t >= 0) {
             const int rank = __popcll(same & lt_mask), group = __popcll(same);
             const int start = cnt_load(&hist[t]);
-            rank_tmp[base_pick + q] = start + rank;         // rank inside this slice
+            r = start + rank;
             if (rank == group - 1) cnt_store(&hist[t], start + group);
         }
         __builtin_amdgcn_wave_barrier();
+        return r;
+    };
+    if (in_regs) {
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c)
+            if (q_begin + c * kWave < q_end) rk[c] = rank_chunk(tk[c]);
+    } else {
+        for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
+            const int q = q0 + lane;
+            const int32_t t = q < q_end ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+            const int r = rank_chunk(t);
+            if (t >= 0) rank_tmp[base_pick + q] = r;
+        }
     }
     __syncthreads();
 
@@ -150,11 +174,17 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
     }
     __syncthreads();
     for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)b * (T + 1) + t] = tok_start[t];
-    for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
-        const int q = q0 + lane;
-        if (q < q_end) {
-            const int32_t t = load_token(Ind, ind_dtype, base_pick + q, T);
-            if (t >= 0) perm[base_pick + tok_start[t] + hist[t] + rank_tmp[base_pick + q]] = q;
+    if (in_regs) {
+#pragma unroll
+        for (int c = 0; c < MAXC; ++c)
+            if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rk[c]] = q_begin + c * kWave + lane;
+    } else {
+        for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
+            const int q = q0 + lane;
+            if (q < q_end) {
+                const int32_t t = load_token(Ind, ind_dtype, base_pick + q, T);
+                if (t >= 0) perm[base_pick + tok_start[t] + hist[t] + rank_tmp[base_pick + q]] = q;
+            }
         }
     }
 }
@@ -235,9 +265,9 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const PT *P, cons
         float acc[VW];
 #pragma unroll
         for (int x = 0; x < VW; ++x) acc[x] = 0.f;
-        for (int s = s0; s < s1; ++s) {
-            const int q = perm[(size_t)b * N + s];
-            const PT *src = P + ((size_t)b * N + q) * I + (size_t)iv * VW;
+        // rows are fetched 4 at a time (their table entries first, then the rows) so that a
+        // short segment costs two memory round trips; they are still added in table order
+        auto add_row = [&](const PT *src) {
             if constexpr (sizeof(PT) == 4) {
                 if constexpr (VW == 4) {
                     f32x4 v = *reinterpret_cast<const f32x4 *>(src);
@@ -258,6 +288,38 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const PT *P, cons
                     uint32_t hbits = (uint32_t)src[0];
                     acc[0] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
                 }
+            }
+        };
+        const int32_t *pb = perm + (size_t)b * N;
+        const PT *Pb = P + (size_t)b * N * I + (size_t)iv * VW;
+        for (int s = s0; s < s1; s += 4) {
+            const int n4 = min(4, s1 - s);
+            int q[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) q[u] = pb[min(s + u, s1 - 1)];
+            if constexpr (VW == 4) {
+                typedef typename std::conditional<sizeof(PT) == 4, f32x4, u32x2>::type vec_t;
+                vec_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    if (u >= n4) break;
+                    if constexpr (sizeof(PT) == 4) {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) acc[x] += v[u][x];
+                    } else {
+#pragma unroll
+                        for (int x = 0; x < 4; ++x) {
+                            uint32_t hbits = (v[u][x >> 1] >> (16 * (x & 1))) & 0xffffu;
+                            acc[x] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
+                        }
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (u < n4) add_row(Pb + (size_t)q[u] * I);
             }
         }
         size_t at = row * I + (size_t)iv * VW;

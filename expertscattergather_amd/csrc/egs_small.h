@@ -52,6 +52,7 @@ struct SmallRowsParams {
     // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
     int32_t csr_blocks;
     int32_t *seg_off, *perm, *rank_tmp;
+    unsigned long long *dbg_times;   // optional [grid*4][2] wall-clock stamps per wavefront (performance debugging)
 };
 
 // Requirements (checked by the launcher): 2-byte elements, R == 32*KS, N % 8 == 0,
@@ -79,6 +80,7 @@ __global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
     const int m0 = (tile * 4 + wave) * 64;
     if (m0 >= Me) return;                       // no barriers below: a wave may leave alone
     const int N = p.N;
+    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)blockIdx.x * 4 + wave) * 2] = wall_clock64();
 
     // Which output column does accumulator row a' = 4g+r of MFMA tile tn hold?  Chosen so that
     // in every store instruction the four lanes g = 0..3 of one result row write one contiguous
@@ -221,6 +223,7 @@ __global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
             }
         }
     }
+    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)blockIdx.x * 4 + wave) * 2 + 1] = wall_clock64();
 }
 
 }  // namespace egs

@@ -96,6 +96,11 @@ const char *egs_last_hip_error(void);
  * specialised small-expert kernels (both must give results within the same tolerances). */
 void egs_set_force_generic(int on);
 
+/* Performance-debugging aid: when `buf` is non-NULL (device memory, 2 x uint64 per wavefront of
+ * the launch, zero-filled by the caller) the small-expert rows kernel stamps the 100 MHz wall
+ * clock at each wavefront's start and end.  NULL switches it off. */
+void egs_set_debug_times(void *buf);
+
 /* bytes of scratch the op needs for these sizes (0 is a valid answer).
  * `mode` is an egs_scatter_mode and only matters for ops that scatter. */
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype);

@@ -1,0 +1,109 @@
+"""The C ABI library loads without a GPU, exports every symbol the header declares, and
+rejects bad arguments before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from expertscattergather_amd import _abi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "egs_hip.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(egs_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not _abi.is_built():
+        from expertscattergather_amd import build
+        build.build()
+    return _abi.lib()
+
+
+def test_header_and_binding_agree(lib):
+    names = declared_functions()
+    assert len(names) >= 12
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in egs_hip.h but not exported"
+    assert sorted(_abi.SIGNATURES) == names, "the ctypes table must list exactly the header's functions"
+
+
+def test_version_and_status_strings(lib):
+    assert lib.egs_abi_version() == _abi.ABI_VERSION == 1
+    assert lib.egs_status_string(0) == b"ok"
+    assert lib.egs_status_string(_abi.EGS_ERR_BAD_DTYPE) == b"Unknown dtype"
+    for code in range(-10, 0):
+        assert lib.egs_status_string(code) not in (b"", b"unknown status")
+    assert lib.egs_status_string(-99) == b"unknown status"
+    assert lib.egs_last_hip_error() == b""
+
+
+def test_enums_match_header():
+    text = open(HEADER).read()
+    for name, value in (("EGS_F32", _abi.F32), ("EGS_F16", _abi.F16), ("EGS_BF16", _abi.BF16),
+                        ("EGS_FP8_E4M3", _abi.FP8_E4M3), ("EGS_IND_I16", _abi.IND_I16), ("EGS_IND_I32", _abi.IND_I32),
+                        ("EGS_IND_I64", _abi.IND_I64), ("EGS_IND_U8", _abi.IND_U8), ("EGS_W_EIJ", _abi.W_EIJ),
+                        ("EGS_W_EJI", _abi.W_EJI), ("EGS_SCATTER_DETERMINISTIC", _abi.SCATTER_DETERMINISTIC),
+                        ("EGS_SCATTER_ATOMIC", _abi.SCATTER_ATOMIC), ("EGS_OP_GATHER_BACKWARD", _abi.OP_GATHER_BACKWARD),
+                        ("EGS_OP_SCATTER_BACKWARD", _abi.OP_SCATTER_BACKWARD), ("EGS_ERR_HIP", _abi.EGS_ERR_HIP)):
+        m = re.search(rf"\b{name}\s*=\s*(-?\d+)", text)
+        assert m and int(m.group(1)) == value, name
+
+
+def test_argument_validation_needs_no_gpu(lib):
+    d = _abi.Dims(2, 8, 3, 4, 16, 8)
+    p = 0x1000  # never dereferenced: every call below must fail validation first
+    g = lib.egs_gather_gemm
+    assert g(None, p, p, p, None, d, 128, 16, 2, 2, 2, 0, None) == -1          # null X
+    assert g(p, p, p, p, None, None, 128, 16, 2, 2, 2, 0, None) == -1          # null dims
+    assert g(p, p, p, p, None, d, 128, 16, 7, 7, 2, 0, None) == -3             # unknown dtype
+    assert g(p, p, p, p, None, d, 128, 16, 2, 2, 9, 0, None) == -3             # unknown index dtype
+    assert g(p, p, p, p, None, d, 128, 16, 2, 2, 2, 5, None) == -4             # unknown layout
+    assert g(p, p, p, p, None, d, 128, 16, 2, 0, 2, 0, None) == -9             # mixed dtypes
+    assert g(p, p, p, p, None, d, 128, 16, 2, 3, 2, 0, None) == -1             # fp8 weights without scales
+    assert g(p, p, p, p, None, d, 128, 8, 2, 2, 2, 0, None) == -10             # token stride < row
+    assert g(p + 1, p, p, p, None, d, 128, 16, 2, 2, 2, 0, None) == -7         # misaligned
+    bad = _abi.Dims(2, 8, -3, 4, 16, 8)
+    assert g(p, p, p, p, None, bad, 128, 16, 2, 2, 2, 0, None) == -2
+    sc = lib.egs_gemm_scatter
+    assert sc(p, p, p, p, p, 1 << 30, d, 2, 2, 1, 7, None) == -5               # unknown mode
+    assert sc(p, p, p, p, None, 0, d, 2, 2, 1, 0, None) == -6                  # workspace missing
+    need = lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, 0, d, 2)
+    assert need > 0
+    assert sc(p, p, p, p, 0x2000, need - 1, d, 2, 2, 1, 0, None) == -6          # workspace too small
+    assert sc(p, p, p, p, 0x2001, need, d, 2, 2, 1, 0, None) == -7              # workspace not 256-byte aligned
+    dw = lib.egs_dw
+    assert dw(p, p, p, None, None, 0, d, 128, 16, 2, 2, 2, 0, None) == -1
+    assert lib.egs_validate_indices(p, 2, -1, 8, p, None) == -2
+    assert lib.egs_validate_indices(None, 2, 4, 8, p, None) == -1
+    # empty problems succeed without any pointer
+    empty = _abi.Dims(0, 8, 3, 4, 16, 8)
+    assert g(None, None, None, None, None, empty, 0, 0, 2, 2, 2, 0, None) == 0
+    assert sc(None, None, None, None, None, 0, empty, 2, 2, 1, 0, None) == 0
+
+
+def test_workspace_sizes_are_consistent(lib):
+    d = _abi.Dims(64, 256, 32, 32, 128, 64)
+    wb = lib.egs_workspace_bytes
+    assert wb(_abi.OP_GATHER_GEMM, 0, d, 2) == 0
+    det, dw = wb(_abi.OP_GEMM_SCATTER, 0, d, 2), wb(_abi.OP_DW, 0, d, 2)
+    assert det >= 64 * 32 * 32 * 128 * 4                                     # fp32 product rows
+    assert wb(_abi.OP_GATHER_BACKWARD, 0, d, 2) == det + dw
+    assert wb(_abi.OP_SCATTER_BACKWARD, 0, d, 2) == dw
+    assert wb(_abi.OP_GEMM_SCATTER, 1, d, 0) == 0                             # fp32 atomic mode adds into the output
+    assert det % 256 == 0 and dw % 256 == 0
+    assert wb(99, 0, d, 2) == 0 and wb(_abi.OP_DW, 0, d, 9) == 0
+
+
+def test_check_raises_like_the_reference():
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        _abi.check(_abi.EGS_ERR_BAD_DTYPE, "x")
+    with pytest.raises(RuntimeError, match="workspace"):
+        _abi.check(-6, "x")
+    _abi.check(0, "x")

@@ -1,0 +1,98 @@
+"""Host-side behaviour that needs no GPU: module construction and parameters, op registration
+with fake implementations, error paths, scatter-mode switch, synthetic workloads."""
+import math
+
+import pytest
+import torch
+
+import expertscattergather_amd as egs
+from expertscattergather_amd import hip_kernels as hk, workloads as wl
+
+
+def test_modules_construct_on_cpu_with_reference_parameter_shapes():
+    g = egs.ExpertGather(5, 12, 7)
+    s = egs.ExpertScatter(5, 7, 12, bias=True)
+    assert g.W.shape == (5, 12, 7) and g.bias is None           # reference egs/torch_interface.py:15-19
+    assert s.W.shape == (5, 7, 12) and s.bias.shape == (5, 1, 12)
+    assert g.W.abs().max() <= 1 / math.sqrt(12) and s.W.abs().max() <= 1 / math.sqrt(12)
+    assert set(g.state_dict()) == {"W"} and set(s.state_dict()) == {"W", "bias"}
+    g2 = egs.ExpertGather(5, 12, 7); g2.load_state_dict(g.state_dict())
+    assert torch.equal(g2.W, g.W)
+    before = g.W
+    assert g.to(torch.bfloat16) is g and g.W.dtype == torch.bfloat16 and g.W is before   # optimizer references survive
+
+
+def test_no_cpu_fallback():
+    g = egs.ExpertGather(2, 8, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        g(torch.randn(1, 3, 8), torch.zeros(1, 2, 2, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        egs.ExpertScatter(2, 4, 8)(torch.randn(1, 2, 2, 4), torch.zeros(1, 2, 2, dtype=torch.int64), 3)
+
+
+def test_ops_are_registered_with_fake_implementations():
+    hk.create_kernels(); hk.create_kernels()                     # idempotent
+    ops = torch.ops.egs_amd
+    X = torch.empty(2, 5, 8, device="meta"); Wg = torch.empty(4, 8, 6, device="meta")
+    Ws = torch.empty(4, 6, 8, device="meta"); Ind = torch.empty(2, 4, 3, dtype=torch.int64, device="meta")
+    Y = ops.expert_gather_forward_call_fn(X, Wg, Ind, torch.float32)
+    assert Y.shape == (2, 4, 3, 6) and Y.dtype == X.dtype
+    dX, dW = ops.expert_gather_backward_call_fn(X, Wg, Ind, Y, torch.float32)
+    assert dX.shape == X.shape and dW.shape == Wg.shape and dX is not X and dW is not Wg
+    out = ops.expert_scatter_forward_call_fn(Y, Ws, Ind, 5, torch.float32)
+    assert out.shape == (2, 5, 8)
+    dY, dWs = ops.expert_scatter_backward_call_fn(Y, Ws, Ind, out, torch.float32)
+    assert dY.shape == Y.shape and dWs.shape == Ws.shape
+    assert hk.expert_gather_forward_call is ops.expert_gather_forward_call_fn
+
+
+def test_autograd_functions_trace_on_meta_tensors():
+    X = torch.empty(2, 5, 8, device="meta", requires_grad=True)
+    W = torch.empty(4, 8, 6, device="meta", requires_grad=True)
+    Ind = torch.empty(2, 4, 3, dtype=torch.int64, device="meta")
+    Y = hk.ExpertGatherFunction.apply(X, W, Ind)
+    Y.sum().backward()
+    assert X.grad.shape == X.shape and W.grad.shape == W.shape
+    Ws = torch.empty(4, 6, 8, device="meta", requires_grad=True)
+    out = hk.ExpertScatterFunction.apply(Y.detach().requires_grad_(True), Ws, Ind, 5)
+    out.sum().backward()
+    assert Ws.grad.shape == Ws.shape
+
+
+def test_dtype_ids_and_errors():
+    assert [hk.dtype_to_type_id(d) for d in (torch.float32, torch.float16, torch.bfloat16)] == [0, 1, 2]
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        hk.dtype_to_type_id(torch.float64)
+
+
+def test_scatter_mode_switch():
+    assert hk.get_scatter_mode() in ("deterministic", "atomic")
+    keep = hk.get_scatter_mode()
+    hk.set_scatter_mode("ATOMIC"); assert hk.get_scatter_mode() == "atomic"
+    with pytest.raises(ValueError):
+        hk.set_scatter_mode("fastest")
+    hk.set_scatter_mode(keep)
+
+
+def test_workloads_follow_the_benchmark_configurations():
+    assert wl.CONFIGS["C2"].dims == (64, 256, 32, 32, 128, 64)
+    assert wl.algorithmic_bytes(wl.CONFIGS["C2"].dims, 2) == 13631488
+    assert wl.algorithmic_bytes(wl.CONFIGS["C1"].dims, 4) == 26738688
+    assert wl.algorithmic_bytes(wl.CONFIGS["C3"].dims, 2) == 270532608
+    assert wl.algorithmic_bytes(wl.CONFIGS["C4"].dims, 2) == 59768832
+    assert wl.algorithmic_bytes(wl.CONFIGS["C5"].dims, 2, 1, fp8_scales=True) == 1078460416
+    assert wl.flops(wl.CONFIGS["C2"].dims) == 2 * 64 * 32 * 32 * 128 * 64
+    inp = wl.make_inputs(wl.CONFIGS["C2"], dims=(3, 40, 4, 8, 16, 8))
+    Ind = inp["Ind"]
+    assert Ind.shape == (3, 4, 8) and Ind.min() >= 0 and Ind.max() < 40
+    for b in range(3):
+        for e in range(4):
+            assert Ind[b, e].unique().numel() == 8             # without replacement per (b, e)
+    again = wl.make_inputs(wl.CONFIGS["C2"], dims=(3, 40, 4, 8, 16, 8))
+    assert all(torch.equal(inp[k], again[k]) for k in inp)       # seeded
+    z = wl.make_inputs(wl.CONFIGS["C4"], dims=(2, 64, 4, 32, 16, 8))["Ind"]
+    assert z.min() >= 0 and z.max() < 64
+    assert max(z[b, e].unique().numel() for b in range(2) for e in range(4)) < 32   # Zipf repeats tokens
+    Wq, scale = wl.quantize_fp8_weights(torch.randn(3, 16, 8))
+    assert Wq.dtype == torch.float8_e4m3fn and scale.shape == (3, 8)
+    assert (Wq.float().abs().amax(dim=1) <= 448).all()
