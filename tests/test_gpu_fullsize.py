@@ -1,0 +1,138 @@
+"""Full-size runs of the benchmark configurations on the GPU.
+
+C1/C2 are compared element by element with the oracle.  C3, C4 and C5 are too large for the
+float64 oracle as a whole, so they are checked (a) against the oracle on slices that are cheap to
+recompute (some (b,e) blocks of the gather, one batch element of the scatter, some experts of
+dW) and (b) through size-independent properties: exact linearity under scaling by 2,
+adjointness of gather and scatter, bitwise repeatability of the deterministic mode, agreement
+of the two scatter modes, rows nobody picks being exactly zero."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import egs_oracle as O
+from tests._util import assert_close, np64
+
+pytestmark = pytest.mark.gpu
+
+from expertscattergather_amd import hip_kernels as hk, workloads as wl
+
+hk.create_kernels()
+DEV = "cuda"
+
+
+def gpu_inputs(name):
+    cfg = wl.CONFIGS[name]
+    inp = wl.make_inputs(cfg)
+    return cfg, inp, {k: v.to(DEV) for k, v in inp.items()}
+
+
+def test_c1_fp32_forward_matches_oracle():
+    cfg, inp, g = gpu_inputs("C1")
+    B, T, E, K, I, J = cfg.dims
+    Y = hk.expert_gather_forward_call(g["X"], g["Wg"], g["Ind"], torch.float32)
+    out = hk.expert_scatter_forward_call(Y, g["Ws"], g["Ind"], T, torch.float32)
+    Indn = inp["Ind"].numpy()
+    assert_close(Y, O.gather_forward(np64(inp["X"]), np64(inp["Wg"]), Indn), torch.float32, "C1 Y")
+    assert_close(out, O.scatter_forward(np64(Y), np64(inp["Ws"]), Indn, T), torch.float32, "C1 out")
+
+
+@pytest.mark.parametrize("mode", ["deterministic", "atomic"])
+def test_c2_bf16_chain_matches_oracle(mode):
+    cfg, inp, g = gpu_inputs("C2")
+    B, T, E, K, I, J = cfg.dims
+    hk.set_scatter_mode(mode)
+    try:
+        Y = hk.expert_gather_forward_call(g["X"], g["Wg"], g["Ind"], torch.float32)
+        out = hk.expert_scatter_forward_call(Y, g["Ws"], g["Ind"], T, torch.float32)
+        dY, dWs = hk.expert_scatter_backward_call(Y, g["Ws"], g["Ind"], g["dOut"], torch.float32)
+        dX, dWg = hk.expert_gather_backward_call(g["X"], g["Wg"], g["Ind"], dY, torch.float32)
+        torch.cuda.synchronize()
+    finally:
+        hk.set_scatter_mode("deterministic")
+    Indn = inp["Ind"].numpy()
+    Xn, Wgn, Wsn, dOn = (np64(inp[k]) for k in ("X", "Wg", "Ws", "dOut"))
+    assert_close(Y, O.gather_forward(Xn, Wgn, Indn), torch.bfloat16, "C2 Y")
+    assert_close(out, O.scatter_forward(np64(Y), Wsn, Indn, T), torch.bfloat16, "C2 out")
+    dYo, dWso = O.scatter_backward(np64(Y), Wsn, Indn, dOn)
+    assert_close(dY, dYo, torch.bfloat16, "C2 dY"); assert_close(dWs, dWso, torch.bfloat16, "C2 dWs")
+    dXo, dWgo = O.gather_backward(Xn, Wgn, Indn, np64(dY))
+    assert_close(dX, dXo, torch.bfloat16, "C2 dX"); assert_close(dWg, dWgo, torch.bfloat16, "C2 dWg")
+
+
+def check_large(name, modes):
+    cfg, inp, g = gpu_inputs(name)
+    B, T, E, K, I, J = cfg.dims
+    X, Wg, Ws, dOut, Ind = (g[k] for k in ("X", "Wg", "Ws", "dOut", "Ind"))
+    Indn = inp["Ind"].numpy()
+    rng = np.random.default_rng(0)
+
+    # ---- gather: slices against the oracle, exact linearity under scaling by 2
+    Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    for b, e in zip(rng.integers(0, B, 4), rng.integers(0, E, 4)):
+        ref = np64(inp["X"][b])[Indn[b, e]] @ np64(inp["Wg"][e])
+        assert_close(Y[b, e], ref, cfg.dtype, f"{name} Y[{b},{e}]")
+    assert torch.equal(hk.expert_gather_forward_call(2 * X, Wg, Ind, torch.float32), 2 * Y)
+
+    # ---- scatter: one batch element against the oracle, modes agree, unpicked rows are zero
+    outs = {}
+    for mode in modes:
+        hk.set_scatter_mode(mode)
+        try:
+            outs[mode] = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+            if mode == "deterministic":
+                assert torch.equal(outs[mode], hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32))
+        finally:
+            hk.set_scatter_mode("deterministic")
+    b = int(rng.integers(0, B))
+    ref = O.scatter_forward(np64(Y[b:b + 1]), np64(inp["Ws"]), Indn[b:b + 1], T, acc=np.float64)
+    picked = torch.zeros(T, dtype=torch.bool); picked[inp["Ind"][b].reshape(-1)] = True
+    for mode, out in outs.items():
+        assert_close(out[b:b + 1], ref, cfg.dtype, f"{name} out[{b}] {mode}")
+        assert (out[b].cpu()[~picked] == 0).all()
+    out = outs[modes[0]]
+
+    # ---- adjointness: <gather(X), G> = <X, scatter_with_Wg(G)>  (fp32 sums of bf16 products)
+    G = torch.randn(B, E, K, J, device=DEV, generator=torch.Generator(DEV).manual_seed(3)).to(cfg.dtype)
+    dXg, dWg = hk.expert_gather_backward_call(X, Wg, Ind, G, torch.float32)
+    lhs = (Y.double() * G.double()).sum().item(); rhs = (X.double() * dXg.double()).sum().item()
+    scale = (Y.double().abs() * G.double().abs()).sum().item()
+    assert abs(lhs - rhs) <= 2e-3 * scale, (lhs, rhs, scale)
+
+    # ---- weight gradients: a few experts against the oracle
+    dYs, dWs = hk.expert_scatter_backward_call(Y, Ws, Ind, dOut, torch.float32)
+    for e in rng.integers(0, E, 2):
+        rows = np.concatenate([np64(inp["X"][bb])[Indn[bb, e]] for bb in range(B)])          # [B*K, I]
+        assert_close(dWg[e], rows.T @ np64(G[:, e]).reshape(B * K, J), cfg.dtype, f"{name} dWg[{e}]")
+        grows = np.concatenate([np64(inp["dOut"][bb])[Indn[bb, e]] for bb in range(B)])
+        assert_close(dWs[e], np64(Y[:, e]).reshape(B * K, J).T @ grows, cfg.dtype, f"{name} dWs[{e}]")
+    b, e = int(rng.integers(0, B)), int(rng.integers(0, E))
+    assert_close(dYs[b, e], np64(inp["dOut"][b])[Indn[b, e]] @ np64(inp["Ws"][e]).T, cfg.dtype, f"{name} dY[{b},{e}]")
+    assert torch.equal(dWg, hk.expert_gather_backward_call(X, Wg, Ind, G, torch.float32)[1])
+
+
+def test_c3_long_sequence_bf16():
+    check_large("C3", ["deterministic"])
+
+
+def test_c4_zipf_routing_both_modes():
+    check_large("C4", ["deterministic", "atomic"])
+
+
+def test_c5_fp8_weights_forward():
+    cfg = wl.CONFIGS["C5"]
+    B, T, E, K, I, J = cfg.dims
+    gen = torch.Generator().manual_seed(cfg.seed)
+    X = torch.randn(B, T, I, generator=gen).to(torch.bfloat16)
+    Ind = wl.uniform_routing(B, T, E, K, gen)
+    Wq = torch.empty(E, I, J, dtype=torch.float8_e4m3fn); scale = torch.empty(E, J)
+    for e0 in range(0, E, 32):                           # quantise in chunks to bound host memory
+        w = torch.randn(32, I, J, generator=gen) / I ** 0.5
+        Wq[e0:e0 + 32], scale[e0:e0 + 32] = wl.quantize_fp8_weights(w)
+    Xg, Wqg, sg, Ig = X.to(DEV), Wq.to(DEV), scale.to(DEV), Ind.to(DEV)
+    Y = hk.expert_gather_fp8w_forward(Xg, Wqg, sg, Ig)
+    rng = np.random.default_rng(1)
+    for b, e in zip(rng.integers(0, B, 4), rng.integers(0, E, 4)):
+        W = O.dequant_fp8_weights(Wq[e:e + 1].view(torch.uint8).numpy(), scale[e:e + 1].numpy())[0]
+        assert_close(Y[b, e], np64(X[b])[Ind[b, e].numpy()] @ W, torch.bfloat16, f"C5 Y[{b},{e}]")
+    assert torch.equal(hk.expert_gather_fp8w_forward(2 * Xg, Wqg, sg, Ig), 2 * Y)
