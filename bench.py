@@ -25,6 +25,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
+# Counters cannot be read from inside this process, so the figure is the recorded one.
+MEASURED_TRAFFIC_BYTES = {("C2", "gather_gemm"): 17342138}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -36,6 +41,8 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="only launch a 64 MiB device copy (3x) and the dominant kernel (5x), for rocprofv3 --pmc runs")
     return ap.parse_args()
 
 
@@ -59,6 +66,18 @@ def main():
     inp = wl.make_inputs(cfg)
     X, Wg, Ws, dOut, Ind = (inp[k].to(dev) for k in ("X", "Wg", "Ws", "dOut", "Ind"))
     fwd_only = args.config in ("C1", "C5")
+
+    if args.pmc_probe:
+        # FETCH_SIZE / WRITE_SIZE calibration: a copy kernel of known size next to the dominant kernel
+        src = torch.empty(64 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        for _ in range(5):
+            hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": True, "copy_bytes_read": 64 << 20, "copy_bytes_written": 64 << 20}))
+        return
 
     def step():
         Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
@@ -204,7 +223,8 @@ def main():
         "kernel_us": {k: round(v[0] * 1e6, 2) for k, v in kernels.items()},
         "kernel_hbm_gbps": {k: round(v[1] / v[0] * 1e-9, 1) for k, v in kernels.items()},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(dom_bytes / dom_s * 1e-9, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
                      "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_s * 1e6, 3)},
         "cpu_baseline": cpu,
     }

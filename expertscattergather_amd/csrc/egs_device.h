@@ -228,4 +228,16 @@ __device__ __forceinline__ bool decode_expert_tile(int bid, int tiles_per_expert
     return e < E;
 }
 
+// The other choice: consecutive row tiles of all experts share an XCD (row tile = 8*group +
+// id % 8), so the source rows of a batch element, which several experts pick, are fetched into
+// one L2 only, at the price of every XCD fetching every W[e].
+__device__ __forceinline__ bool decode_tile_expert(int bid, int tiles_per_expert, int E, int &e, int &tile)
+{
+    int xcd = bid & 7, slot = bid >> 3;
+    int tg = slot / E;
+    e = slot - tg * E;
+    tile = tg * 8 + xcd;
+    return tile < tiles_per_expert;
+}
+
 }  // namespace egs

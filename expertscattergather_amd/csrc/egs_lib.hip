@@ -211,7 +211,7 @@ constexpr uint64_t kSpan32 = 0xFFFFFFFFull;      // the small kernel addresses w
 template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
 int launch_rows_small_ks(SmallRowsParams &p, int R, size_t lds, hipStream_t s)
 {
-    const int grid = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
+    const int grid = (p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e) + p.csr_blocks;
     p.dbg_times = g_dbg_times;
     switch (R) {
     case 32: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
@@ -254,7 +254,14 @@ int try_gather_small(const void *X, const void *W, const void *Ind, void *Y, con
     p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
     p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
     p.tiles_per_e = (int)((Me + 255) / 256);
-    if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e > INT32_MAX) return 1;
+    if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX) return 1;
+    {   // which operand is worth keeping XCD-local: the source rows (each read by ~E*K/T experts) or W[e]
+        const double picks_per_token = (double)d->E * d->K / d->T;
+        const double x_bytes = (double)d->B * d->T * R * 2, w_bytes = (double)d->E * R * N * 2;
+        const double by_expert = x_bytes * (picks_per_token < 8 ? (picks_per_token < 1 ? 1 : picks_per_token) : 8) + w_bytes;
+        const double by_rows = x_bytes + w_bytes * (p.tiles_per_e < 8 ? p.tiles_per_e : 8);
+        p.rows_share_xcd = by_rows < by_expert;
+    }
     const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
     return act_dtype == EGS_BF16 ? launch_rows_small<ElemBF16, true, false>(p, R, nmajor, 0, s)
                                  : launch_rows_small<ElemF16, true, false>(p, R, nmajor, 0, s);

@@ -49,6 +49,7 @@ struct SmallRowsParams {
     int64_t lda_b, lda_t;
     int32_t ind_dtype;
     int32_t tiles_per_e;    // workgroups (256 picks each) per expert
+    int32_t rows_share_xcd; // 1: row tiles map to XCDs (source rows reused across experts), 0: experts map to XCDs
     // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
     int32_t csr_blocks;
     int32_t *seg_off, *perm, *rank_tmp;
@@ -73,7 +74,9 @@ __global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
         }
     }
     int e, tile;
-    if (!decode_expert_tile((int)blockIdx.x - (GATHER ? 0 : p.csr_blocks), p.tiles_per_e, p.E, e, tile)) return;
+    const int bid = (int)blockIdx.x - (GATHER ? 0 : p.csr_blocks);
+    if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
+                         : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
