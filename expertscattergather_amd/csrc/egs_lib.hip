@@ -192,69 +192,49 @@ int launch_rows_gemm(RowsGemmParams &p, int act_dtype, bool w_trans, hipStream_t
 }
 
 // ------------------------------------------------------------------------------ small-expert fast paths
-size_t device_lds_limit()
-{
-    static size_t limit = 0;
-    if (limit == 0) {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) == hipSuccess && v > 0)
-            limit = (size_t)v;
-        else
-            limit = 64 * 1024;
-    }
-    return limit;
-}
+constexpr uint64_t kSpan32 = 0xFFFFFFFFull;      // the small kernels address with 32-bit byte offsets
 
-constexpr uint64_t kSpan32 = 0xFFFFFFFFull;      // the small kernel addresses with 32-bit byte offsets
-
-template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
-int launch_rows_small_ks(SmallRowsParams &p, int R, size_t lds, hipStream_t s)
-{
-    const int grid = (p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e) + p.csr_blocks;
-    p.dbg_times = g_dbg_times;
-    switch (R) {
-    case 32: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
-    case 64: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
-    default: hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, 4, TN, GATHER, OUT_F32>), dim3(grid), dim3(kThreads), lds, s, p); break;
-    }
-    EGS_CHECK_LAUNCH("rows_small_kernel");
-    return EGS_OK;
-}
-
-template <class TT, bool GATHER, bool OUT_F32>
-int launch_rows_small(SmallRowsParams &p, int R, bool nmajor, size_t lds, hipStream_t s)
-{
-    if (p.N <= 64)
-        return nmajor ? launch_rows_small_ks<TT, true, 4, GATHER, OUT_F32>(p, R, lds, s)
-                      : launch_rows_small_ks<TT, false, 4, GATHER, OUT_F32>(p, R, lds, s);
-    return nmajor ? launch_rows_small_ks<TT, true, 8, GATHER, OUT_F32>(p, R, lds, s)
-                  : launch_rows_small_ks<TT, false, 8, GATHER, OUT_F32>(p, R, lds, s);
-}
+// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
+size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
 
 bool small_shape_ok(int act_dtype, int R, int N)
 {
     return act_dtype != EGS_F32 && (R == 32 || R == 64 || R == 128) && N % 8 == 0 && N >= 8 && N <= 128;
 }
 
-// Both return 1 if the problem does not qualify (caller takes the general kernel), else a status.
-int try_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
-                     int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, hipStream_t s)
+// one launch of rows_small_kernel, or its share of a heterogeneous launch
+struct SmallRowsJob {
+    SmallRowsParams p;
+    int R, act_dtype, blocks;
+    bool nmajor, gather, out_f32;
+    size_t lds;
+};
+// one launch of dw_small_kernel (or its share of a heterogeneous launch) plus the second pass
+struct SmallDwJob {
+    SmallDwParams q;
+    int blocks, act_dtype;
+    size_t w_elems;
+    bool done;          // set once the first pass has been enqueued
+};
+
+bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
+                       int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, SmallRowsJob &j)
 {
     const int R = d->I, N = d->J;
-    if (w_dtype != act_dtype || !small_shape_ok(act_dtype, R, N)) return 1;
-    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16)) return 1;
-    if ((ldx_b * 2) % 16 || (ldx_t * 2) % 16 || d->T == 0) return 1;
+    if (g_force_generic || w_dtype != act_dtype || !small_shape_ok(act_dtype, R, N)) return false;
+    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16)) return false;
+    if ((ldx_b * 2) % 16 || (ldx_t * 2) % 16 || d->T == 0) return false;
     const int64_t Me = (int64_t)d->B * d->K;
+    if (Me == 0 || d->E == 0) return false;
     const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + R) * 2;
-    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32 || (uint64_t)Me * d->E * N * 2 > kSpan32) return 1;
-    SmallRowsParams p;
-    memset(&p, 0, sizeof(p));
+    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32 || (uint64_t)Me * d->E * N * 2 > kSpan32) return false;
+    memset(&j, 0, sizeof(j));
+    SmallRowsParams &p = j.p;
     p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y;
     p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
     p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
     p.tiles_per_e = (int)((Me + 255) / 256);
-    if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX) return 1;
+    if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return false;
     {   // which operand is worth keeping XCD-local: the source rows (each read by ~E*K/T experts) or W[e]
         const double picks_per_token = (double)d->E * d->K / d->T;
         const double x_bytes = (double)d->B * d->T * R * 2, w_bytes = (double)d->E * R * N * 2;
@@ -262,44 +242,129 @@ int try_gather_small(const void *X, const void *W, const void *Ind, void *Y, con
         const double by_rows = x_bytes + w_bytes * (p.tiles_per_e < 8 ? p.tiles_per_e : 8);
         p.rows_share_xcd = by_rows < by_expert;
     }
-    const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
-    return act_dtype == EGS_BF16 ? launch_rows_small<ElemBF16, true, false>(p, R, nmajor, 0, s)
-                                 : launch_rows_small<ElemF16, true, false>(p, R, nmajor, 0, s);
+    j.R = R; j.act_dtype = act_dtype; j.gather = true; j.out_f32 = false; j.lds = 0;
+    j.nmajor = (w_layout == EGS_W_EIJ);                 // [E,I,J] = [E,R,N]
+    j.blocks = p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e;
+    return true;
 }
 
-// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
-size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
-
-// product rows of the scatter in pick order; when `csr` is set the routing table is built by
-// extra workgroups of the same launch
-int try_scatter_rows_small(const void *Y, const void *W, void *rows, bool rows_f32, const egs_dims *d, int act_dtype,
-                           int w_layout, bool csr, const void *Ind, int ind_dtype, int32_t *seg_off, int32_t *perm,
-                           int32_t *rank_tmp, hipStream_t s)
+// product rows of the scatter in pick order; with `ride` the routing table is built by extra
+// workgroups of the same launch
+bool make_scatter_rows_small(const void *Y, const void *W, void *rows, bool rows_f32, const egs_dims *d, int act_dtype,
+                             int w_layout, bool ride, const void *Ind, int ind_dtype, int32_t *seg_off, int32_t *perm,
+                             int32_t *rank_tmp, SmallRowsJob &j)
 {
     const int R = d->J, N = d->I;
-    if (!small_shape_ok(act_dtype, R, N)) return 1;
-    if (!aligned_to(Y, 16) || !aligned_to(W, 16)) return 1;
+    if (g_force_generic || !small_shape_ok(act_dtype, R, N)) return false;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16)) return false;
     const int64_t Me = (int64_t)d->B * d->K;
+    if (Me == 0 || d->E == 0) return false;
     if ((uint64_t)Me * d->E * R * 2 > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32 ||
-        (uint64_t)Me * d->E * N * 4 > kSpan32) return 1;
-    SmallRowsParams p;
-    memset(&p, 0, sizeof(p));
+        (uint64_t)Me * d->E * N * 4 > kSpan32) return false;
+    memset(&j, 0, sizeof(j));
+    SmallRowsParams &p = j.p;
     p.A = (const char *)Y; p.W = (const char *)W; p.C = (char *)rows;
     p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
     p.tiles_per_e = (int)((Me + 255) / 256);
-    size_t lds = 0;
-    if (csr) {
+    if (ride) {
         p.csr_blocks = d->B; p.Ind = Ind; p.ind_dtype = ind_dtype;
         p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp;
-        lds = csr_count_lds(d->T, 4);
+        j.lds = csr_count_lds(d->T, 4);
     }
-    if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e + p.csr_blocks > INT32_MAX) return 1;
-    const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
-    if (act_dtype == EGS_BF16)
-        return rows_f32 ? launch_rows_small<ElemBF16, false, true>(p, R, nmajor, lds, s)
-                        : launch_rows_small<ElemBF16, false, false>(p, R, nmajor, lds, s);
-    return rows_f32 ? launch_rows_small<ElemF16, false, true>(p, R, nmajor, lds, s)
-                    : launch_rows_small<ElemF16, false, false>(p, R, nmajor, lds, s);
+    if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e + p.csr_blocks > INT32_MAX / 2) return false;
+    j.R = R; j.act_dtype = act_dtype; j.gather = false; j.out_f32 = rows_f32;
+    j.nmajor = (w_layout == EGS_W_EJI);                 // [E,J,I] = [E,R,N]
+    j.blocks = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
+    return true;
+}
+
+bool make_dw_small(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
+                   int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout,
+                   const DwPlan &pl, SmallDwJob &j)
+{
+    if (!pl.small_ok || g_force_generic || d->T == 0) return false;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * 2;
+    if (!aligned_to(Xs, 16) || !aligned_to(Ys, 16) || !aligned_to(dW, 16) || (ldx_b * 2) % 16 || (ldx_t * 2) % 16) return false;
+    if (x_span > kSpan32 || (uint64_t)d->B * d->E * d->K * d->J * 2 > kSpan32) return false;
+    if ((int64_t)8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S > INT32_MAX / 2) return false;
+    memset(&j, 0, sizeof(j));
+    SmallDwParams &q = j.q;
+    q.Xs = (const char *)Xs; q.Ys = (const char *)Ys; q.Ind = Ind; q.part = (float *)workspace; q.dW = (char *)dW;
+    q.B = d->B; q.T = d->T; q.E = d->E; q.K = d->K; q.I = d->I; q.J = d->J;
+    q.ldx_b = ldx_b; q.ldx_t = ldx_t; q.ind_dtype = ind_dtype;
+    q.i_tiles = pl.s_i_tiles; q.j_tiles = pl.s_j_tiles; q.S = pl.s_S; q.rows_per_split = pl.s_rows_per_split;
+    q.out_dtype = out_dtype; q.dw_layout = dw_layout;
+    j.blocks = 8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S;
+    j.act_dtype = act_dtype;
+    j.w_elems = (size_t)d->E * d->I * d->J;
+    return true;
+}
+
+// ---- launch of a rows job, alone or sharing the launch with the first pass of a dW job
+template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
+int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+{
+    j.p.dbg_times = g_dbg_times;
+    if (dw != nullptr) {
+        hipLaunchKernelGGL((rows_dw_small_kernel<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>), dim3(j.blocks + dw->blocks),
+                           dim3(kThreads), j.lds, s, j.p, dw->q, j.blocks);
+        dw->done = true;
+    } else {
+        hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>), dim3(j.blocks), dim3(kThreads),
+                           j.lds, s, j.p);
+    }
+    EGS_CHECK_LAUNCH("rows_small_kernel");
+    return EGS_OK;
+}
+
+template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
+int launch_rows_small_ks(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+{
+    switch (j.R) {
+    case 32: return launch_rows_small_one<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>(j, dw, s);
+    case 64: return launch_rows_small_one<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>(j, dw, s);
+    default: return launch_rows_small_one<TT, W_NMAJOR, 4, TN, GATHER, OUT_F32>(j, dw, s);
+    }
+}
+
+template <class TT, bool GATHER, bool OUT_F32>
+int launch_rows_small_tn(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+{
+    if (j.p.N <= 64)
+        return j.nmajor ? launch_rows_small_ks<TT, true, 4, GATHER, OUT_F32>(j, dw, s)
+                        : launch_rows_small_ks<TT, false, 4, GATHER, OUT_F32>(j, dw, s);
+    return j.nmajor ? launch_rows_small_ks<TT, true, 8, GATHER, OUT_F32>(j, dw, s)
+                    : launch_rows_small_ks<TT, false, 8, GATHER, OUT_F32>(j, dw, s);
+}
+
+template <class TT>
+int launch_rows_small_tt(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+{
+    if (j.gather) return launch_rows_small_tn<TT, true, false>(j, dw, s);
+    return j.out_f32 ? launch_rows_small_tn<TT, false, true>(j, dw, s) : launch_rows_small_tn<TT, false, false>(j, dw, s);
+}
+
+int launch_rows_small_job(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+{
+    return j.act_dtype == EGS_BF16 ? launch_rows_small_tt<ElemBF16>(j, dw, s) : launch_rows_small_tt<ElemF16>(j, dw, s);
+}
+
+int launch_dw_small_alone(SmallDwJob &j, hipStream_t s)
+{
+    if (j.act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_small_kernel<ElemBF16>, dim3(j.blocks), dim3(kThreads), 0, s, j.q);
+    else hipLaunchKernelGGL(dw_small_kernel<ElemF16>, dim3(j.blocks), dim3(kThreads), 0, s, j.q);
+    EGS_CHECK_LAUNCH("dw_small_kernel");
+    j.done = true;
+    return EGS_OK;
+}
+
+int launch_dw_reduce4(const SmallDwJob &j, hipStream_t s)
+{
+    if (j.q.S <= 1) return EGS_OK;
+    hipLaunchKernelGGL(dw_reduce4_kernel, dim3(grid_1d(j.w_elems / 4, 2048)), dim3(kThreads), 0, s,
+                       (const float *)j.q.part, j.q.dW, j.q.S, j.w_elems / 4, j.q.out_dtype);
+    EGS_CHECK_LAUNCH("dw_reduce4_kernel");
+    return EGS_OK;
 }
 
 // routing table of the deterministic scatter as a launch of its own: counting sort with
@@ -344,15 +409,52 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
     return EGS_OK;
 }
 
+// fixed-order reduction of the product rows per token; when `reduce` is given (and qualifies) the
+// second pass of that weight gradient shares the launch
+int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, const int32_t *perm, void *Out,
+                       const egs_dims *d, int act_dtype, SmallDwJob *reduce, hipStream_t s)
+{
+    const int N = d->E * d->K;
+    const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
+    const int iv = vw4 ? d->I / 4 : d->I;
+    SegSumParams sp;
+    memset(&sp, 0, sizeof(sp));
+    sp.P = rows; sp.seg_off = seg_off; sp.perm = perm; sp.out = (char *)Out;
+    sp.B = d->B; sp.T = d->T; sp.N = N; sp.I = d->I;
+    while ((1 << sp.tpr_log2) < iv && sp.tpr_log2 < 8) ++sp.tpr_log2;      // threads sharing an output row (<= 256)
+    sp.gx = ceil_div(d->T, kThreads >> sp.tpr_log2);
+    sp.gy = d->B;
+    while ((int64_t)sp.gx * sp.gy > (1 << 22)) sp.gy = (sp.gy + 1) / 2;     // stride loop over batch elements beyond that
+    const int seg_blocks = sp.gx * sp.gy;
+    const bool fuse = reduce != nullptr && reduce->done && reduce->q.S > 1 && vw4;
+    const int red_blocks = fuse ? grid_1d(reduce->w_elems / 4, 1024) : 0;
+#define EGS_SEGSUM(TT, PT)                                                                                                  \
+    do {                                                                                                                    \
+        if (fuse) hipLaunchKernelGGL((segsum_dwreduce_kernel<TT, PT, 4>), dim3(seg_blocks + red_blocks), dim3(kThreads), 0, \
+                                     s, sp, seg_blocks, (const float *)reduce->q.part, reduce->q.dW, reduce->q.S,           \
+                                     reduce->w_elems / 4, reduce->q.out_dtype);                                             \
+        else if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 4>), dim3(seg_blocks), dim3(kThreads), 0, s, sp);      \
+        else hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 1>), dim3(seg_blocks), dim3(kThreads), 0, s, sp);               \
+    } while (0)
+    if (act_dtype == EGS_F32) EGS_SEGSUM(ElemF32, float);
+    else if (act_dtype == EGS_F16) { if (rows_f32) EGS_SEGSUM(ElemF16, float); else EGS_SEGSUM(ElemF16, uint16_t); }
+    else { if (rows_f32) EGS_SEGSUM(ElemBF16, float); else EGS_SEGSUM(ElemBF16, uint16_t); }
+#undef EGS_SEGSUM
+    EGS_CHECK_LAUNCH("segment_sum_kernel");
+    if (fuse) reduce->q.S = 1;              // second pass done
+    return EGS_OK;
+}
+
 // ------------------------------------------------------------------------------ implementations
 int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
                      const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
                      int w_layout, hipStream_t s)
 {
     const int ES = elem_size(act_dtype), WES = elem_size(w_dtype);
-    if (w_scale == nullptr && !g_force_generic) {
-        int rc = try_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, s);
-        if (rc != 1) return rc;
+    if (w_scale == nullptr) {
+        SmallRowsJob j;
+        if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j))
+            return launch_rows_small_job(j, nullptr, s);
     }
     RowsGemmParams p;
     memset(&p, 0, sizeof(p));
@@ -373,8 +475,11 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
     return launch_rows_gemm<true, EPI_STORE>(p, act_dtype, w_trans, s);
 }
 
+// `dw` (optional): a weight gradient of the same call whose first pass may share the product
+// launch and whose second pass may share the reduction launch
 int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, void *workspace,
-                      const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode, hipStream_t s)
+                      const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode, SmallDwJob *dw,
+                      hipStream_t s)
 {
     const int ES = elem_size(act_dtype);
     const size_t out_elems = (size_t)d->B * d->T * d->I;
@@ -412,88 +517,35 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     int32_t *cnt = d->T > kCsrLdsTokens ? (int32_t *)(ws + pl.cnt_at) : nullptr;
     void *rows = ws + pl.rows_at;
     bool rows_f32 = (mode == EGS_SCATTER_DETERMINISTIC);
-    int rc = 1;
-    if (!g_force_generic && N > 0) {
-        // small experts: the sort rides along with the product when its histograms are small
-        const bool ride = csr_count_lds(d->T, 4) <= 16 * 1024 && N <= 4096;
+    // small experts: the sort rides along with the product when its histograms are small
+    const bool ride = csr_count_lds(d->T, 4) <= 16 * 1024 && N <= 4096 && N > 0;
+    SmallRowsJob j;
+    int rc;
+    if (N > 0 && make_scatter_rows_small(Y, W, rows, rows_f32, d, act_dtype, w_layout, ride, Ind, ind_dtype, seg_off, perm,
+                                         rank_tmp, j)) {
         if (!ride) {
             rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
             if (rc != EGS_OK) return rc;
         }
-        rc = try_scatter_rows_small(Y, W, rows, rows_f32, d, act_dtype, w_layout, ride, Ind, ind_dtype, seg_off, perm,
-                                    rank_tmp, s);
-        if (rc == 1 && ride) {
-            rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
-            if (rc != EGS_OK) return rc;
-            rc = 1;
-        }
+        rc = launch_rows_small_job(j, dw, s);
     } else {
         rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
         if (rc != EGS_OK) return rc;
-        rc = 1;
-    }
-    if (rc == 1) {
         rows_f32 = true;                    // the general kernel writes fp32 rows
         p.C = (char *)rows;
         p.c_vec = d->I % 4 == 0;
         rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
     }
     if (rc != EGS_OK) return rc;
-    const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
-    const size_t items = (size_t)d->B * d->T * (vw4 ? d->I / 4 : d->I);
-    const int grid = grid_1d(items, 65536);
-#define EGS_SEGSUM(TT, PT)                                                                                          \
-    do {                                                                                                            \
-        if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 4>), dim3(grid), dim3(kThreads), 0, s,              \
-                                    (const PT *)rows, seg_off, perm, (char *)Out, d->B, d->T, N, d->I);             \
-        else hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 1>), dim3(grid), dim3(kThreads), 0, s,                  \
-                                (const PT *)rows, seg_off, perm, (char *)Out, d->B, d->T, N, d->I);                 \
-    } while (0)
-    if (act_dtype == EGS_F32) EGS_SEGSUM(ElemF32, float);
-    else if (act_dtype == EGS_F16) { if (rows_f32) EGS_SEGSUM(ElemF16, float); else EGS_SEGSUM(ElemF16, uint16_t); }
-    else { if (rows_f32) EGS_SEGSUM(ElemBF16, float); else EGS_SEGSUM(ElemBF16, uint16_t); }
-#undef EGS_SEGSUM
-    EGS_CHECK_LAUNCH("segment_sum_kernel");
-    return EGS_OK;
+    return launch_segment_sum(rows, rows_f32, seg_off, perm, Out, d, act_dtype, dw, s);
 }
 
-int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
-            int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout, hipStream_t s)
+int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
+               int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout,
+               const DwPlan &pl, hipStream_t s)
 {
     const size_t w_elems = (size_t)d->E * d->I * d->J;
-    if (w_elems == 0) return EGS_OK;
-    const int ES = elem_size(act_dtype), OES = elem_size(out_dtype);
-    const DwPlan pl = plan_dw(d, act_dtype);
-    if (pl.small_ok && !g_force_generic) {
-        const uint64_t x_span = d->T > 0 ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * 2 : 0;
-        const bool ok = d->T > 0 && aligned_to(Xs, 16) && aligned_to(Ys, 16) && aligned_to(dW, 16) && (ldx_b * 2) % 16 == 0 &&
-                        (ldx_t * 2) % 16 == 0 && x_span <= kSpan32 &&
-                        (uint64_t)d->B * d->E * d->K * d->J * 2 <= kSpan32 &&
-                        (int64_t)8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S <= INT32_MAX;
-        if (ok) {
-            SmallDwParams q;
-            memset(&q, 0, sizeof(q));
-            q.Xs = (const char *)Xs; q.Ys = (const char *)Ys; q.Ind = Ind; q.part = (float *)workspace; q.dW = (char *)dW;
-            q.B = d->B; q.T = d->T; q.E = d->E; q.K = d->K; q.I = d->I; q.J = d->J;
-            q.ldx_b = ldx_b; q.ldx_t = ldx_t; q.ind_dtype = ind_dtype;
-            q.i_tiles = pl.s_i_tiles; q.j_tiles = pl.s_j_tiles; q.S = pl.s_S; q.rows_per_split = pl.s_rows_per_split;
-            q.out_dtype = out_dtype; q.dw_layout = dw_layout;
-            const int grid = 8 * ceil_div(d->E, 8) * pl.s_i_tiles * pl.s_j_tiles * pl.s_S;
-            if (act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_small_kernel<ElemBF16>, dim3(grid), dim3(kThreads), 0, s, q);
-            else hipLaunchKernelGGL(dw_small_kernel<ElemF16>, dim3(grid), dim3(kThreads), 0, s, q);
-            EGS_CHECK_LAUNCH("dw_small_kernel");
-            if (pl.s_S > 1) {
-                if (dw_layout == EGS_W_EIJ && w_elems % 4 == 0)
-                    hipLaunchKernelGGL(dw_reduce4_kernel, dim3(grid_1d(w_elems / 4, 2048)), dim3(kThreads), 0, s,
-                                       (const float *)workspace, (char *)dW, pl.s_S, w_elems / 4, out_dtype);
-                else
-                    hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s,
-                                       (const float *)workspace, (char *)dW, pl.s_S, d->E, d->I, d->J, out_dtype, dw_layout);
-                EGS_CHECK_LAUNCH("dw_reduce_kernel");
-            }
-            return EGS_OK;
-        }
-    }
+    const int ES = elem_size(act_dtype);
     DwParams p;
     memset(&p, 0, sizeof(p));
     p.Xs = (const char *)Xs; p.Ys = (const char *)Ys; p.Ind = Ind;
@@ -504,7 +556,6 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
     p.x_vec = aligned_to(Xs, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
     p.y_vec = aligned_to(Ys, 16) && ((int64_t)d->J * ES) % 16 == 0;
     p.o_vec = aligned_to(dW, 16) && d->J % 4 == 0;
-    (void)OES;
     p.i_tiles = pl.i_tiles; p.j_tiles = pl.j_tiles; p.S = pl.S; p.rows_per_split = pl.rows_per_split;
     p.out_dtype = out_dtype; p.dw_layout = dw_layout;
     const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.i_tiles * pl.j_tiles * pl.S;
@@ -521,6 +572,20 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
         EGS_CHECK_LAUNCH("dw_reduce_kernel");
     }
     return EGS_OK;
+}
+
+int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
+            int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout, hipStream_t s)
+{
+    if ((size_t)d->E * d->I * d->J == 0) return EGS_OK;
+    const DwPlan pl = plan_dw(d, act_dtype);
+    SmallDwJob j;
+    if (make_dw_small(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, j)) {
+        int rc = launch_dw_small_alone(j, s);
+        if (rc != EGS_OK) return rc;
+        return launch_dw_reduce4(j, s);
+    }
+    return dw_general(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, s);
 }
 
 // ------------------------------------------------------------------------------ validation
@@ -654,7 +719,7 @@ int egs_gemm_scatter(const void *Y, const void *W, const void *Ind, void *Out,
 {
     int rc = validate_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, act_dtype, ind_dtype, w_layout, mode);
     if (rc != EGS_OK) return rc;
-    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, act_dtype, ind_dtype, w_layout, mode, (hipStream_t)stream);
+    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, act_dtype, ind_dtype, w_layout, mode, nullptr, (hipStream_t)stream);
 }
 
 int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
@@ -695,10 +760,22 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     void *ws2 = workspace ? (char *)workspace + ws_scatter : nullptr;
     rc = validate_dw(X, grad_Y, Ind, grad_W, ws2, ws_dw, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ);
     if (rc != EGS_OK) return rc;
-    // grad_X[b,t,i] = sum_picks sum_j grad_Y[b,e,k,j] * W[e,i,j]
-    rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, (hipStream_t)stream);
+    // grad_X[b,t,i] = sum_picks sum_j grad_Y[b,e,k,j] * W[e,i,j];  grad_W[e,i,j] = sum X[b,Ind,i] * grad_Y[b,e,k,j].
+    // The two are independent: for small experts the weight gradient shares the scatter's launches.
+    hipStream_t s = (hipStream_t)stream;
+    const size_t w_elems = (size_t)d->E * d->I * d->J;
+    const DwPlan dpl = plan_dw(d, dtype);
+    SmallDwJob dwj;
+    const bool dw_small = w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype,
+                                                       EGS_W_EIJ, dpl, dwj);
+    rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr, s);
     if (rc != EGS_OK) return rc;
-    return dw_impl(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, (hipStream_t)stream);
+    if (w_elems == 0) return EGS_OK;
+    if (dw_small) {
+        if (!dwj.done) { rc = launch_dw_small_alone(dwj, s); if (rc != EGS_OK) return rc; }
+        return launch_dw_reduce4(dwj, s);       // no-op when the reduction launch already did it
+    }
+    return dw_general(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dpl, s);
 }
 
 int egs_expert_scatter_forward(const void *Y, const void *W, const void *Ind, void *Out,
@@ -719,15 +796,27 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
     rc = validate_dw(grad_Out, Y, Ind, grad_W, workspace, workspace_bytes, d, ldg_b, ldg_t, dtype, dtype, ind_dtype,
                      EGS_W_EJI);
     if (rc != EGS_OK) return rc;
-    // grad_Y[b,e,k,j] = sum_i grad_Out[b,Ind,i] * W[e,j,i]
-    if ((size_t)d->B * d->E * d->K * d->J > 0) {
-        rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI,
-                              (hipStream_t)stream);
+    // grad_Y[b,e,k,j] = sum_i grad_Out[b,Ind,i] * W[e,j,i];  grad_W[e,j,i] = sum grad_Out[b,Ind,i] * Y[b,e,k,j].
+    // Independent of each other: for small experts they share one launch.
+    hipStream_t s = (hipStream_t)stream;
+    const size_t y_elems = (size_t)d->B * d->E * d->K * d->J, w_elems = (size_t)d->E * d->I * d->J;
+    const DwPlan dpl = plan_dw(d, dtype);
+    SmallRowsJob gj;
+    SmallDwJob dwj;
+    const bool g_small = y_elems > 0 && make_gather_small(grad_Out, W, Ind, grad_Y, d, ldg_b, ldg_t, dtype, dtype, ind_dtype,
+                                                          EGS_W_EJI, gj);
+    const bool dw_small = w_elems > 0 && make_dw_small(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype,
+                                                       ind_dtype, EGS_W_EJI, dpl, dwj);
+    if (g_small && dw_small) {
+        rc = launch_rows_small_job(gj, &dwj, s);
+        if (rc != EGS_OK) return rc;
+        return launch_dw_reduce4(dwj, s);
+    }
+    if (y_elems > 0) {
+        rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);
         if (rc != EGS_OK) return rc;
     }
-    // grad_W[e,j,i] = sum_{b,k} grad_Out[b,Ind,i] * Y[b,e,k,j]
-    return dw_impl(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI,
-                   (hipStream_t)stream);
+    return dw_impl(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);
 }
 
 int egs_validate_indices(const void *Ind, int ind_dtype, int64_t n, int32_t T, int32_t *d_bad_count, void *stream)

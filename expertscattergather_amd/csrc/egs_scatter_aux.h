@@ -250,17 +250,31 @@ __global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t
 // (rows perm[b][s] of P[b], seg_off[t] <= s < seg_off[t+1]); every row of out is written
 // exactly once (tokens nobody picked become zero).  P rows hold PT (float, or 16-bit values
 // of the element type TT); VW elements per thread.
+struct SegSumParams {
+    const void *P;              // product rows [B, N, I], fp32 or 16-bit
+    const int32_t *seg_off, *perm;
+    char *out;                  // [B, T, I]
+    int32_t B, T, N, I;
+    int32_t tpr_log2;           // 2^tpr_log2 threads share an output row
+    int32_t gx, gy;             // logical grid: gx row groups x gy batch slots
+};
+
 template <class TT, class PT, int VW>
-__global__ __launch_bounds__(kThreads) void segment_sum_kernel(const PT *P, const int32_t *seg_off, const int32_t *perm,
-                                                               char *out, int32_t B, int32_t T, int32_t N, int32_t I)
+__device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const int bx, const int by)
 {
+    // 2^tpr_log2 threads share an output row (VW columns each, looping if the row is wider);
+    // bx selects a group of rows of batch element by (+ a stride loop over b)
+    const PT *P = reinterpret_cast<const PT *>(sp.P);
+    const int32_t *seg_off = sp.seg_off, *perm = sp.perm;
+    char *out = sp.out;
+    const int B = sp.B, T = sp.T, N = sp.N, I = sp.I, tpr_log2 = sp.tpr_log2;
     const int IV = (I + VW - 1) / VW;
-    const size_t items = (size_t)B * T * IV;
-    for (size_t item = (size_t)blockIdx.x * kThreads + threadIdx.x; item < items;
-         item += (size_t)gridDim.x * kThreads) {
-        size_t row = item / IV;
-        int iv = (int)(item - row * IV);
-        int b = (int)(row / T), t = (int)(row - (size_t)b * T);
+    const int tpr = 1 << tpr_log2;
+    const int t = bx * (kThreads >> tpr_log2) + ((int)threadIdx.x >> tpr_log2);
+    if (t >= T) return;
+    for (int b = by; b < B; b += sp.gy)
+    for (int iv = (int)threadIdx.x & (tpr - 1); iv < IV; iv += tpr) {
+        const size_t row = (size_t)b * T + t;
         int s0 = seg_off[(size_t)b * (T + 1) + t], s1 = seg_off[(size_t)b * (T + 1) + t + 1];
         float acc[VW];
 #pragma unroll
@@ -339,6 +353,12 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(const PT *P, cons
             }
         }
     }
+}
+
+template <class TT, class PT, int VW>
+__global__ __launch_bounds__(kThreads) void segment_sum_kernel(SegSumParams sp)
+{
+    segment_sum_body<TT, PT, VW>(sp, (int)blockIdx.x % sp.gx, (int)blockIdx.x / sp.gx);
 }
 
 // zero n floats (the atomic mode's accumulator).  A kernel rather than a memset so that the

@@ -59,22 +59,21 @@ struct SmallRowsParams {
 // Requirements (checked by the launcher): 2-byte elements, R == 32*KS, N % 8 == 0,
 // 8 <= N <= 16*TN, A rows / W / C 16-byte aligned, every tensor smaller than 4 GiB.
 template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
-__global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
+__device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const int block, int32_t *sh_cnt_small)
 {
     constexpr int TQ = 4;                       // 4 row tiles = 64 picks per wave
     constexpr int R = 32 * KS;
     constexpr int OES = OUT_F32 ? 4 : 2;        // output element size
     static_assert(!(GATHER && OUT_F32), "gather results are stored in the element type");
     if constexpr (!GATHER) {
-        if ((int)blockIdx.x < p.csr_blocks) {
-            extern __shared__ int32_t sh_cnt_small[];
-            csr_count_body(sh_cnt_small, (int)blockIdx.x, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
+        if (block < p.csr_blocks) {
+            csr_count_body(sh_cnt_small, block, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
                            p.E * p.K, p.seg_off, p.perm, p.rank_tmp);
             return;
         }
     }
     int e, tile;
-    const int bid = (int)blockIdx.x - (GATHER ? 0 : p.csr_blocks);
+    const int bid = block - (GATHER ? 0 : p.csr_blocks);
     if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
                          : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -83,7 +82,7 @@ __global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
     const int m0 = (tile * 4 + wave) * 64;
     if (m0 >= Me) return;                       // no barriers below: a wave may leave alone
     const int N = p.N;
-    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)blockIdx.x * 4 + wave) * 2] = wall_clock64();
+    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)block * 4 + wave) * 2] = wall_clock64();
 
     // Which output column does accumulator row a' = 4g+r of MFMA tile tn hold?  Chosen so that
     // in every store instruction the four lanes g = 0..3 of one result row write one contiguous
@@ -226,7 +225,14 @@ __global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
             }
         }
     }
-    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)blockIdx.x * 4 + wave) * 2 + 1] = wall_clock64();
+    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)block * 4 + wave) * 2 + 1] = wall_clock64();
+}
+
+template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
+__global__ __launch_bounds__(kThreads) void rows_small_kernel(SmallRowsParams p)
+{
+    extern __shared__ int32_t sh_dyn_small[];
+    rows_small_body<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>(p, (int)blockIdx.x, sh_dyn_small);
 }
 
 }  // namespace egs
@@ -260,7 +266,7 @@ constexpr int kDwSmallMaxRows = 1024;   // picks of one workgroup (row offsets s
 // Requirements: 2-byte elements, I % 8 == 0, J % 8 == 0, rows 16-byte aligned, spans < 4 GiB,
 // rows_per_split <= kDwSmallMaxRows.
 template <class TT>
-__global__ __launch_bounds__(kThreads) void dw_small_kernel(SmallDwParams p)
+__device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int block)
 {
     __shared__ __attribute__((aligned(16))) float red[4 * 64 * 64];       // 64 KB: one tile per wavefront
     uint32_t *xoff_lds = reinterpret_cast<uint32_t *>(red);              // reused before the reduction:
@@ -268,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void dw_small_kernel(SmallDwParams p)
 
     int e, tile;
     const int tiles_per_e = p.i_tiles * p.j_tiles * p.S;
-    if (!decode_expert_tile((int)blockIdx.x, tiles_per_e, p.E, e, tile)) return;
+    if (!decode_expert_tile(block, tiles_per_e, p.E, e, tile)) return;
     const int s = tile / (p.i_tiles * p.j_tiles);
     const int ij = tile - s * (p.i_tiles * p.j_tiles);
     const int it = ij / p.j_tiles, jt = ij - it * p.j_tiles;
@@ -356,48 +362,62 @@ __global__ __launch_bounds__(kThreads) void dw_small_kernel(SmallDwParams p)
         }
     __syncthreads();
 
+    // sum the four wavefront tiles in wavefront order and write 4 consecutive elements of the
+    // requested layout per thread: [.,I,J] rows of j, or [.,J,I] rows of i (read transposed from LDS).
+    // Partial sums (S > 1) use the same layout as the final tensor, so the second pass is a plain
+    // element-wise sum.
     const bool direct = (p.S == 1);
+    const bool eji = p.dw_layout != 0;
     for (int item = tid; item < 64 * 16; item += kThreads) {
-        const int i = item >> 4, chunk = item & 15;
-        const int phys = (chunk ^ (i >> 2)) * 4;
-        f32x4 v = *reinterpret_cast<const f32x4 *>(red + i * 64 + phys);
+        const int major = item >> 4, minor4 = (item & 15) * 4;      // major: i (EIJ) or j (EJI); minor: 4 x j or 4 x i
+        f32x4 v;
+        if (!eji) {
+            const int phys = ((minor4 >> 2) ^ (major >> 2)) * 4;
+            v = *reinterpret_cast<const f32x4 *>(red + major * 64 + phys);
 #pragma unroll
-        for (int w = 1; w < 4; ++w) {
-            const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * 4096 + i * 64 + phys);
-            v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
-        }
-        const int gi = i0 + i, gj = j0 + chunk * 4;
-        if (gi >= p.I || gj >= p.J) continue;           // J % 4 == 0: a chunk is inside or outside
-        if (!direct) {
-            *reinterpret_cast<f32x4 *>(p.part + (((size_t)s * p.E + e) * p.I + gi) * p.J + gj) = v;
-        } else if (p.dw_layout == 0) {                  // [E,I,J]
-            const size_t at = ((size_t)e * p.I + gi) * p.J + gj;
-            if (p.out_dtype == 0) {
-                *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.dW) + at) = v;
-            } else {
-                u32x2 w2;
-                w2[0] = p.out_dtype == 1 ? pack2<ElemF16>(v[0], v[1]) : pack2<ElemBF16>(v[0], v[1]);
-                w2[1] = p.out_dtype == 1 ? pack2<ElemF16>(v[2], v[3]) : pack2<ElemBF16>(v[2], v[3]);
-                *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.dW) + at) = w2;
+            for (int w = 1; w < 4; ++w) {
+                const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * 4096 + major * 64 + phys);
+                v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
             }
-        } else {                                        // [E,J,I]
+        } else {
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                const size_t at = ((size_t)e * p.J + gj + x) * p.I + gi;
-                if (p.out_dtype == 0) reinterpret_cast<float *>(p.dW)[at] = v[x];
-                else reinterpret_cast<uint16_t *>(p.dW)[at] =
-                    (uint16_t)(p.out_dtype == 1 ? f32_to_f16_bits(v[x]) : f32_to_bf16_bits(v[x]));
+                const int i = minor4 + x;
+                const int at = i * 64 + (((major >> 2) ^ (i >> 2)) * 4) + (major & 3);
+                float acc1 = red[at];
+#pragma unroll
+                for (int w = 1; w < 4; ++w) acc1 += red[w * 4096 + at];
+                v[x] = acc1;
             }
+        }
+        const int gi = i0 + (eji ? minor4 : major), gj = j0 + (eji ? major : minor4);
+        if (gi >= p.I || gj >= p.J) continue;           // I % 4 == 0 and J % 4 == 0: a group of 4 is inside or outside
+        const size_t at = eji ? ((size_t)e * p.J + gj) * p.I + gi : ((size_t)e * p.I + gi) * p.J + gj;
+        if (!direct) {
+            *reinterpret_cast<f32x4 *>(p.part + (size_t)s * p.E * p.I * p.J + at) = v;
+        } else if (p.out_dtype == 0) {
+            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.dW) + at) = v;
+        } else {
+            u32x2 w2;
+            w2[0] = p.out_dtype == 1 ? pack2<ElemF16>(v[0], v[1]) : pack2<ElemBF16>(v[0], v[1]);
+            w2[1] = p.out_dtype == 1 ? pack2<ElemF16>(v[2], v[3]) : pack2<ElemBF16>(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.dW) + at) = w2;
         }
     }
 }
 
-// dW(e,i,j) = sum_s part[s][e][i][j] in increasing s, rounded once; [E,I,J] output, 4 elements
-// per thread (total % 4 == 0, 16-byte aligned).  The transposed layout uses dw_reduce_kernel.
-__global__ __launch_bounds__(kThreads) void dw_reduce4_kernel(const float *part, char *dW, int32_t S, size_t total4,
-                                                              int32_t out_dtype)
+template <class TT>
+__global__ __launch_bounds__(kThreads) void dw_small_kernel(SmallDwParams p)
 {
-    for (size_t o = (size_t)blockIdx.x * kThreads + threadIdx.x; o < total4; o += (size_t)gridDim.x * kThreads) {
+    dw_small_body<TT>(p, (int)blockIdx.x);
+}
+
+// dW = sum_s part[s] in increasing s, rounded once; partials already have the output's layout.
+// 4 elements per thread (total % 4 == 0, 16-byte aligned); `block` of `nblocks` workgroups.
+__device__ __forceinline__ void dw_reduce4_body(const float *part, char *dW, int32_t S, size_t total4, int32_t out_dtype,
+                                                const int block, const int nblocks)
+{
+    for (size_t o = (size_t)block * kThreads + threadIdx.x; o < total4; o += (size_t)nblocks * kThreads) {
         f32x4 v = reinterpret_cast<const f32x4 *>(part)[o];
         for (int s = 1; s < S; ++s) {
             const f32x4 u = reinterpret_cast<const f32x4 *>(part)[(size_t)s * total4 + o];
@@ -412,6 +432,36 @@ __global__ __launch_bounds__(kThreads) void dw_reduce4_kernel(const float *part,
             reinterpret_cast<u32x2 *>(dW)[o] = w2;
         }
     }
+}
+
+
+__global__ __launch_bounds__(kThreads) void dw_reduce4_kernel(const float *part, char *dW, int32_t S, size_t total4,
+                                                              int32_t out_dtype)
+{
+    dw_reduce4_body(part, dW, S, total4, out_dtype, (int)blockIdx.x, (int)gridDim.x);
+}
+
+// ------------------------------------------------------------------------------------------
+// Heterogeneous launches: independent pieces of one backward call share a launch, so that the
+// call pays one launch ramp and the pieces overlap.  Workgroups [0, rows_blocks) run the rows
+// product (and, for the scatter, the routing table), the rest the weight gradient.
+template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
+__global__ __launch_bounds__(kThreads) void rows_dw_small_kernel(SmallRowsParams p, SmallDwParams q, int rows_blocks)
+{
+    extern __shared__ int32_t sh_dyn_fused[];
+    if ((int)blockIdx.x < rows_blocks) rows_small_body<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>(p, (int)blockIdx.x, sh_dyn_fused);
+    else dw_small_body<TT>(q, (int)blockIdx.x - rows_blocks);
+}
+
+// segment sums of a scatter and the second pass of a weight gradient in one launch:
+// workgroups [0, seg_blocks) reduce product rows per token, the rest sum dW partials
+template <class TT, class PT, int VW>
+__global__ __launch_bounds__(kThreads) void segsum_dwreduce_kernel(SegSumParams sp, int seg_blocks, const float *part,
+                                                                   char *dW, int32_t S, size_t total4, int32_t out_dtype)
+{
+    const int block = (int)blockIdx.x;
+    if (block < seg_blocks) segment_sum_body<TT, PT, VW>(sp, block % sp.gx, block / sp.gx);
+    else dw_reduce4_body(part, dW, S, total4, out_dtype, block - seg_blocks, (int)gridDim.x - seg_blocks);
 }
 
 }  // namespace egs
