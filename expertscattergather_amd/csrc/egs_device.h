@@ -104,15 +104,20 @@ template <> __device__ __forceinline__ void mma_chunk<ElemF32>(f32x4 &acc, const
 }
 
 // ---------------------------------------------------------------------------- index decode
-// Ind is read in its own integer width and never narrowed; returns -1 for out-of-range.
+// Ind is read in its own integer width and never narrowed.  Branch-free for every width (so that
+// several index loads can be in flight): one 8-byte load of the aligned window that contains the
+// element, then shift and sign- or zero-extend.  The window never leaves the allocation because
+// device allocations start and end on multiples of 8 bytes and elements are naturally aligned.
 __device__ __forceinline__ int64_t load_index_raw(const void *ind, int ind_dtype, int64_t at)
 {
-    switch (ind_dtype) {
-    case 0: return (int64_t) reinterpret_cast<const int16_t *>(ind)[at];
-    case 1: return (int64_t) reinterpret_cast<const int32_t *>(ind)[at];
-    case 2: return reinterpret_cast<const int64_t *>(ind)[at];
-    default: return (int64_t) reinterpret_cast<const uint8_t *>(ind)[at];
-    }
+    const int es_log2 = (0x0321 >> (4 * ind_dtype)) & 0xF;          // int16 -> 1, int32 -> 2, int64 -> 3, uint8 -> 0
+    const uint64_t addr = reinterpret_cast<uint64_t>(ind) + ((uint64_t)at << es_log2);
+    uint64_t w = *reinterpret_cast<const uint64_t *>(addr & ~7ull);
+    const int bits = 8 << es_log2;
+    w <<= 64 - bits - (int)(addr & 7ull) * 8;                       // element now in the top `bits` bits
+    const int64_t sx = (int64_t)w >> (64 - bits);                   // sign-extended
+    const int64_t zx = (int64_t)(w >> (64 - bits));                 // zero-extended (uint8)
+    return ind_dtype == 3 ? zx : sx;
 }
 __device__ __forceinline__ int32_t load_token(const void *ind, int ind_dtype, int64_t at, int32_t T)
 {

@@ -375,11 +375,19 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
 {
     const int64_t N = (int64_t)d->E * d->K;
     if (N >= 1) {
+        // as many wavefronts as the per-wavefront histograms leave room for (up to 144 KB of LDS)
+        const size_t budget = 144 * 1024;
         int nw = (int)((N + 63) / 64);
         if (nw > 16) nw = 16;
-        while (nw > 1 && csr_count_lds(d->T, nw) > 64 * 1024) nw >>= 1;
+        while (nw > 1 && csr_count_lds(d->T, nw) > budget) nw >>= 1;
         const size_t lds = csr_count_lds(d->T, nw);
-        if (lds <= 64 * 1024 && (nw > 1 || N <= 4096)) {
+        if (lds <= budget) {
+            static size_t configured = 64 * 1024;
+            if (lds > configured) {
+                hipError_t err = hipFuncSetAttribute((const void *)csr_count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(csr_count_kernel)");
+                configured = lds;
+            }
             hipLaunchKernelGGL(csr_count_kernel, dim3(d->B), dim3(64 * nw), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, rank_tmp);
             EGS_CHECK_LAUNCH("csr_count_kernel");
             return EGS_OK;

@@ -96,7 +96,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
                                                int32_t *perm, int32_t *rank_tmp)
 {
-    constexpr int MAXC = 4;                             // 64-pick chunks whose tokens and ranks stay in registers
+    constexpr int MAXC = 8;                             // 64-pick chunks whose tokens (and ranks) are held in registers at a time
     const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
     int32_t *hist = sh_cnt + (size_t)wave * T;          // this wavefront's counters
     int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
@@ -110,7 +110,8 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int q = q_begin + c * kWave + lane;
-        tk[c] = (in_regs && q < q_end) ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+        const int32_t t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);     // unconditional: loads overlap
+        tk[c] = (in_regs && q < q_end) ? t : -1;
         rk[c] = 0;
     }
 
@@ -141,11 +142,20 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
         for (int c = 0; c < MAXC; ++c)
             if (q_begin + c * kWave < q_end) rk[c] = rank_chunk(tk[c]);
     } else {
-        for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
-            const int q = q0 + lane;
-            const int32_t t = q < q_end ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
-            const int r = rank_chunk(t);
-            if (t >= 0) rank_tmp[base_pick + q] = r;
+        // long slices: MAXC chunks of tokens in flight at a time, ranks parked in global scratch
+        for (int q0 = q_begin; q0 < q_end; q0 += MAXC * kWave) {
+#pragma unroll
+            for (int c = 0; c < MAXC; ++c) {
+                const int q = q0 + c * kWave + lane;
+                const int32_t t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);
+                tk[c] = q < q_end ? t : -1;
+            }
+#pragma unroll
+            for (int c = 0; c < MAXC; ++c) {
+                if (q0 + c * kWave >= q_end) break;
+                const int r = rank_chunk(tk[c]);
+                if (tk[c] >= 0) rank_tmp[base_pick + q0 + c * kWave + lane] = r;
+            }
         }
     }
     __syncthreads();
@@ -161,16 +171,29 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
         tok_start[t] = run;
     }
     __syncthreads();
-    if (wave == 0) {                                        // exclusive scan of the totals over tokens
+    {   // exclusive scan of the totals over tokens: each wavefront scans a contiguous part,
+        // then the parts are offset by the totals of the parts before them
+        __shared__ int32_t part_total[16];
+        const int tw = ((T + NW - 1) / NW + 63) & ~63;
+        const int t_begin = wave * tw, t_end = min(T, t_begin + tw);
         int running = 0;
-        for (int t0 = 0; t0 < T; t0 += kWave) {
+        for (int t0 = t_begin; t0 < t_end; t0 += kWave) {
             const int t = t0 + lane;
-            const int c = t < T ? tok_start[t] : 0;
+            const int c = t < t_end ? tok_start[t] : 0;
             const int incl = wave_inclusive_scan(c, lane);
-            if (t < T) tok_start[t] = running + incl - c;
+            if (t < t_end) tok_start[t] = running + incl - c;
             running += __shfl(incl, kWave - 1, kWave);
         }
-        if (lane == 0) tok_start[T] = running;
+        if (lane == 0) part_total[wave] = running;
+        __syncthreads();
+        int before = 0, total = 0;
+        for (int w = 0; w < NW; ++w) {
+            const int c = part_total[w];
+            if (w < wave) before += c;
+            total += c;
+        }
+        for (int t = t_begin + lane; t < t_end; t += kWave) tok_start[t] += before;
+        if (tid == 0) tok_start[T] = total;
     }
     __syncthreads();
     for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)b * (T + 1) + t] = tok_start[t];
@@ -179,12 +202,18 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
         for (int c = 0; c < MAXC; ++c)
             if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rk[c]] = q_begin + c * kWave + lane;
     } else {
-        for (int q0 = q_begin; q0 < q_end; q0 += kWave) {
-            const int q = q0 + lane;
-            if (q < q_end) {
-                const int32_t t = load_token(Ind, ind_dtype, base_pick + q, T);
-                if (t >= 0) perm[base_pick + tok_start[t] + hist[t] + rank_tmp[base_pick + q]] = q;
+        for (int q0 = q_begin; q0 < q_end; q0 += MAXC * kWave) {
+            int32_t rr[MAXC];
+#pragma unroll
+            for (int c = 0; c < MAXC; ++c) {
+                const int q = q0 + c * kWave + lane;
+                const int32_t t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);
+                rr[c] = rank_tmp[base_pick + min(q, N - 1)];
+                tk[c] = q < q_end ? t : -1;
             }
+#pragma unroll
+            for (int c = 0; c < MAXC; ++c)
+                if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rr[c]] = q0 + c * kWave + lane;
         }
     }
 }
@@ -306,35 +335,46 @@ __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const i
         };
         const int32_t *pb = perm + (size_t)b * N;
         const PT *Pb = P + (size_t)b * N * I + (size_t)iv * VW;
-        for (int s = s0; s < s1; s += 4) {
-            const int n4 = min(4, s1 - s);
-            int q[4];
+        int s = s0;
+        if constexpr (VW == 4) {
+            typedef typename std::conditional<sizeof(PT) == 4, f32x4, u32x2>::type vec_t;
+            auto add_vec = [&](const vec_t &v) {
+                if constexpr (sizeof(PT) == 4) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) q[u] = pb[min(s + u, s1 - 1)];
-            if constexpr (VW == 4) {
-                typedef typename std::conditional<sizeof(PT) == 4, f32x4, u32x2>::type vec_t;
+                    for (int x = 0; x < 4; ++x) acc[x] += v[x];
+                } else {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        uint32_t hbits = (v[x >> 1] >> (16 * (x & 1))) & 0xffffu;
+                        acc[x] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
+                    }
+                }
+            };
+            // long segments (hot tokens): 16 rows in flight per thread; added in table order all the same
+            for (; s + 16 <= s1; s += 16) {
+                int q[16];
+                vec_t v[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) q[u] = pb[s + u];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
+#pragma unroll
+                for (int u = 0; u < 16; ++u) add_vec(v[u]);
+            }
+            for (; s < s1; s += 4) {
+                const int n4 = min(4, s1 - s);
+                int q[4];
                 vec_t v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) q[u] = pb[min(s + u, s1 - 1)];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    if (u >= n4) break;
-                    if constexpr (sizeof(PT) == 4) {
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) acc[x] += v[u][x];
-                    } else {
-#pragma unroll
-                        for (int x = 0; x < 4; ++x) {
-                            uint32_t hbits = (v[u][x >> 1] >> (16 * (x & 1))) & 0xffffu;
-                            acc[x] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
-                        }
-                    }
-                }
-            } else {
-#pragma unroll
                 for (int u = 0; u < 4; ++u)
-                    if (u < n4) add_row(Pb + (size_t)q[u] * I);
+                    if (u < n4) add_vec(v[u]);
             }
+        } else {
+            for (; s < s1; ++s) add_row(Pb + (size_t)pb[s] * I);
         }
         size_t at = row * I + (size_t)iv * VW;
         if constexpr (TT::ES == 4) {
