@@ -187,6 +187,42 @@ __device__ __forceinline__ u32x4 load_chunk_fp8_as_bf16(const char *row, int k0,
     return fp8x8_to_bf16_chunk(lo, hi);
 }
 
+// 4 consecutive 16-bit elements (8 bytes) with the same guards as load_chunk; `vec_ok` = the row
+// start is 8-byte aligned and k0 is a multiple of 4.
+__device__ __forceinline__ u32x2 load_half_chunk16(const char *row, int k0, int klim, bool vec_ok)
+{
+    u32x2 v = {0u, 0u};
+    if (row == nullptr || k0 >= klim) return v;
+    if (vec_ok && k0 + 4 <= klim) return *reinterpret_cast<const u32x2 *>(row + (size_t)k0 * 2);
+    const uint16_t *p = reinterpret_cast<const uint16_t *>(row) + k0;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+        uint32_t h = (k0 + x < klim) ? (uint32_t)p[x] : 0u;
+        v[x >> 1] |= h << (16 * (x & 1));
+    }
+    return v;
+}
+// 4 consecutive fp8 (e4m3fn) bytes -> 4 bf16; `vec_ok` = 4-byte aligned row start, k0 % 4 == 0.
+__device__ __forceinline__ u32x2 load_half_chunk_fp8_as_bf16(const char *row, int k0, int klim, bool vec_ok)
+{
+    u32x2 z = {0u, 0u};
+    if (row == nullptr || k0 >= klim) return z;
+    uint32_t w = 0;
+    if (vec_ok && k0 + 4 <= klim) {
+        w = *reinterpret_cast<const uint32_t *>(row + k0);
+    } else {
+        const uint8_t *p = reinterpret_cast<const uint8_t *>(row) + k0;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) w |= ((k0 + x < klim) ? (uint32_t)p[x] : 0u) << (8 * x);
+    }
+    auto a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    auto b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    u32x2 v;
+    v[0] = (f32_bits(a[0]) >> 16) | (f32_bits(a[1]) & 0xffff0000u);
+    v[1] = (f32_bits(b[0]) >> 16) | (f32_bits(b[1]) & 0xffff0000u);
+    return v;
+}
+
 // ---------------------------------------------------------------------------- LDS tile
 // A tile holds ROWS rows of BK reduction elements, K-major (a row's chunks are adjacent), so
 // an MFMA operand fragment is one 16-byte LDS read per lane.  Chunk positions inside each
@@ -213,6 +249,18 @@ __device__ __forceinline__ void transpose8x8_16b(const u32x4 (&in)[8], u32x4 (&o
         }
     }
 }
+// 8 rows x 4 columns of 16-bit values (in[x] = 4 columns of row x) -> out[c] = the 8 rows of column c
+__device__ __forceinline__ void transpose8x4_16b(const u32x2 (&in)[8], u32x4 (&out)[4])
+{
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            uint32_t lo = in[2 * p][c >> 1], hi = in[2 * p + 1][c >> 1];
+            out[c][p] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        }
+}
+
 __device__ __forceinline__ void transpose4x4_32b(const u32x4 (&in)[4], u32x4 (&out)[4])
 {
 #pragma unroll

@@ -154,20 +154,32 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
     const int Me = p.B * p.K;
     if (Me == 0 || p.E == 0 || p.N == 0) return EGS_OK;
     const int e_groups = ceil_div(p.E, 8);
+    // tile shape: 128 x 64 for narrow outputs, 256 x 256 (8 wavefronts) when the product is large
+    // enough to be bound by operand traffic (16-bit types), else 128 x 128
+    const bool big = TT::ES == 2 && EPI != EPI_ATOMIC_F32 && p.N >= 192 && Me >= 512 && p.R >= 128;
     if (p.N <= 64) {
         constexpr int BM = 128, BN = 64;
         p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
         int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
         if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
         hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 4, 1, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
-                           dim3(kThreads), 0, s, p);
+                           dim3(256), 0, s, p);
+    } else if (big) {
+        if constexpr (TT::ES == 2 && EPI != EPI_ATOMIC_F32) {
+            constexpr int BM = 256, BN = 256;
+            p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
+            int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
+            if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+            hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 4, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
+                               dim3(512), 0, s, p);
+        }
     } else {
         constexpr int BM = 128, BN = 128;
         p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
         int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
         if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
         hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
-                           dim3(kThreads), 0, s, p);
+                           dim3(256), 0, s, p);
     }
     EGS_CHECK_LAUNCH("rows_gemm_kernel");
     return EGS_OK;
@@ -474,7 +486,7 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
     const bool w_trans = (w_layout == EGS_W_EIJ);       // [E,I,J]: the reduction index selects the row
     p.a_vec = aligned_to(X, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
     const int64_t w_row = w_trans ? d->J : d->I;
-    p.w_vec = WES == 1 ? (aligned_to(W, 8) && w_row % 8 == 0) : (aligned_to(W, 16) && (w_row * WES) % 16 == 0);
+    p.w_vec = WES == 1 ? (aligned_to(W, 8) && w_row % 8 == 0) : (aligned_to(W, 16) && (w_row * WES) % 16 == 0);   // stricter than the 8-byte blocks of the transposed loader need
     p.c_vec = aligned_to(Y, 16) && d->J % 4 == 0;
     if (w_dtype == EGS_FP8_E4M3) {
         return w_trans ? launch_rows_gemm_cfg<ElemBF16, 1, true, true, EPI_STORE>(p, s)

@@ -6,7 +6,8 @@
 // where m = b*K + k enumerates the picks of one expert e.  One workgroup owns a BM x BN tile
 // of one expert's product, stages BK-wide slabs of both operands in K-major swizzled LDS
 // tiles (register prefetch of the next slab overlaps the MFMAs of the current one) and runs
-// 16x16 MFMA tiles on 4 wavefronts.
+// 16x16 MFMA tiles on WM x WN wavefronts (4 for the 128-wide tiles, 8 for the 256 x 256 tile
+// whose higher reuse matters once both operands stream through L2).
 //
 // Replaces the reference's expert_gather_kernel (egs/triton_kernels.py:49-143) and
 // expert_scatter_kernel (:156-247).  Unlike those, the M dimension of a tile is the picks of
@@ -34,17 +35,17 @@ struct RowsGemmParams {
 };
 
 template <class TT, int WES, int BM, int BN, int BK, int WM, int WN, bool GATHER, bool W_TRANS, int EPI>
-__global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
+__global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmParams p)
 {
+    constexpr int NT = WM * WN * kWave;          // threads per workgroup: one wavefront per (WM, WN) cell
     constexpr int ES = TT::ES, VEC = TT::VEC;
     constexpr int CH = BK / VEC;                 // chunks per LDS row
     constexpr int KSTEPS = CH / 4;               // MFMA chunk steps per slab
     constexpr bool SWAP = (EPI == EPI_ATOMIC_F32);   // atomics want consecutive n across lanes
     constexpr int TM = BM / WM / 16, TN = BN / WN / 16;
     constexpr bool W_FP8 = (WES == 1);
-    static_assert(WM * WN == kThreads / kWave, "wave grid must cover the workgroup");
-    static_assert(BM <= kThreads, "row bookkeeping uses one thread per tile row");
-    static_assert((BM * CH) % kThreads == 0 && kThreads % CH == 0, "M loader mapping");
+    static_assert(BM <= NT, "row bookkeeping uses one thread per tile row");
+    static_assert((BM * CH) % NT == 0 && NT % CH == 0, "M loader mapping");
     static_assert(!W_FP8 || TT::ES == 2, "fp8 weights are widened to bf16");
 
     __shared__ __attribute__((aligned(16))) char smem_m[BM * BK * ES];
@@ -62,16 +63,19 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
     const bool w_vec = p.w_vec != 0, a_vec = p.a_vec != 0;
 
     // ---------------- weight-side loader
-    constexpr int NVN = (BN * CH + kThreads - 1) / kThreads;            // K-major: chunks per thread
-    constexpr int KB = BK / VEC, NBK = BN / VEC;                        // transposed: VEC x VEC blocks
-    constexpr int NBL = (KB * NBK + kThreads - 1) / kThreads;
-    u32x4 nreg[W_TRANS ? NBL * VEC : NVN];
+    constexpr int NVN = (BN * CH + NT - 1) / NT;            // K-major: chunks per thread
+    // transposed: blocks of VEC reduction rows x BW output columns (16-bit: 8 x 4 so that every
+    // thread gets one block and holds 16 registers of it; fp32: 4 x 4)
+    constexpr int BW = 4;
+    constexpr int KB = BK / VEC, NBK = BN / BW;
+    constexpr int NBL = (KB * NBK + NT - 1) / NT;
+    u32x4 nreg[W_TRANS ? (VEC == 8 ? NBL * 4 : NBL * VEC) : NVN];     // 16-bit blocks: 8 x u32x2 packed in 4 x u32x4
 
     auto issue_n = [&](int kt) {
         if constexpr (!W_TRANS) {
 #pragma unroll
             for (int i = 0; i < NVN; ++i) {
-                int v = tid + i * kThreads;
+                int v = tid + i * NT;
                 int row = v / CH, c = v % CH;
                 int n = n0 + row;
                 const char *ptr = (v < BN * CH && n < N) ? We + (size_t)n * R * WES : nullptr;
@@ -81,14 +85,21 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
         } else {
 #pragma unroll
             for (int i = 0; i < NBL; ++i) {
-                int blk = tid + i * kThreads;
+                int blk = tid + i * NT;
                 int kb = blk / NBK, nb = blk % NBK;
 #pragma unroll
                 for (int r = 0; r < VEC; ++r) {
                     int rr = kt * BK + kb * VEC + r;
                     const char *ptr = (blk < KB * NBK && rr < R) ? We + (size_t)rr * N * WES : nullptr;
-                    if constexpr (W_FP8) nreg[i * VEC + r] = load_chunk_fp8_as_bf16(ptr, n0 + nb * VEC, N, w_vec);
-                    else nreg[i * VEC + r] = load_chunk<ES>(ptr, n0 + nb * VEC, N, w_vec);
+                    if constexpr (VEC == 8) {
+                        u32x2 h;
+                        if constexpr (W_FP8) h = load_half_chunk_fp8_as_bf16(ptr, n0 + nb * BW, N, w_vec);
+                        else h = load_half_chunk16(ptr, n0 + nb * BW, N, w_vec);
+                        nreg[i * 4 + (r >> 1)][(r & 1) * 2] = h[0];
+                        nreg[i * 4 + (r >> 1)][(r & 1) * 2 + 1] = h[1];
+                    } else {
+                        nreg[i * VEC + r] = load_chunk<ES>(ptr, n0 + nb * BW, N, w_vec);
+                    }
                 }
             }
         }
@@ -98,21 +109,30 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
         if constexpr (!W_TRANS) {
 #pragma unroll
             for (int i = 0; i < NVN; ++i) {
-                int v = tid + i * kThreads;
+                int v = tid + i * NT;
                 if (v < BN * CH) tile_n[tile_chunk_index<CH>(v / CH, v % CH)] = nreg[i];
             }
         } else {
 #pragma unroll
             for (int i = 0; i < NBL; ++i) {
-                int blk = tid + i * kThreads;
+                int blk = tid + i * NT;
                 int kb = blk / NBK, nb = blk % NBK;
                 if (blk < KB * NBK) {
-                    u32x4 in[VEC], out[VEC];
+                    u32x4 out[4];
+                    if constexpr (VEC == 8) {
+                        u32x2 in[8];
 #pragma unroll
-                    for (int r = 0; r < VEC; ++r) in[r] = nreg[i * VEC + r];
-                    if constexpr (VEC == 8) transpose8x8_16b(in, out); else transpose4x4_32b(in, out);
+                        for (int r = 0; r < 8; ++r)
+                            in[r] = u32x2{nreg[i * 4 + (r >> 1)][(r & 1) * 2], nreg[i * 4 + (r >> 1)][(r & 1) * 2 + 1]};
+                        transpose8x4_16b(in, out);
+                    } else {
+                        u32x4 in[4];
 #pragma unroll
-                    for (int c = 0; c < VEC; ++c) tile_n[tile_chunk_index<CH>(nb * VEC + c, kb)] = out[c];
+                        for (int r = 0; r < 4; ++r) in[r] = nreg[i * VEC + r];
+                        transpose4x4_32b(in, out);
+                    }
+#pragma unroll
+                    for (int c = 0; c < BW; ++c) tile_n[tile_chunk_index<CH>(nb * BW + c, kb)] = out[c];
                 }
             }
         }
@@ -148,13 +168,13 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
     __syncthreads();
 
     // ---------------- row-side loader (K-major source rows)
-    constexpr int NVM = BM * CH / kThreads;
+    constexpr int NVM = BM * CH / NT;
     const int mc = tid % CH;
     const char *mrow[NVM];
     u32x4 mreg[NVM];
 #pragma unroll
     for (int i = 0; i < NVM; ++i) {
-        int64_t ao = a_off[tid / CH + i * (kThreads / CH)];
+        int64_t ao = a_off[tid / CH + i * (NT / CH)];
         mrow[i] = ao < 0 ? nullptr : p.A + ao * ES;
     }
     auto issue_m = [&](int kt) {
@@ -164,7 +184,7 @@ __global__ __launch_bounds__(kThreads) void rows_gemm_kernel(RowsGemmParams p)
     auto commit_m = [&]() {
         u32x4 *tile_m = reinterpret_cast<u32x4 *>(smem_m);
 #pragma unroll
-        for (int i = 0; i < NVM; ++i) tile_m[tile_chunk_index<CH>(tid / CH + i * (kThreads / CH), mc)] = mreg[i];
+        for (int i = 0; i < NVM; ++i) tile_m[tile_chunk_index<CH>(tid / CH + i * (NT / CH), mc)] = mreg[i];
     };
     issue_m(0);
 

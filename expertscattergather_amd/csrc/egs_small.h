@@ -28,18 +28,6 @@
 
 namespace egs {
 
-// 8 rows x 4 columns of 16-bit values (in[x] = 4 columns of row x) -> out[c] = the 8 rows of column c
-__device__ __forceinline__ void transpose8x4_16b(const u32x2 (&in)[8], u32x4 (&out)[4])
-{
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            uint32_t lo = in[2 * p][c >> 1], hi = in[2 * p + 1][c >> 1];
-            out[c][p] = (c & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-        }
-}
-
 struct SmallRowsParams {
     const char *A;          // GATHER: [B,T,R] rows, strides (lda_b, lda_t, 1) elements;  else [B,E,K,R] dense
     const char *W;          // [E,R,N] (W_NMAJOR) or [E,N,R]
