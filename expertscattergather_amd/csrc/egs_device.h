@@ -223,6 +223,54 @@ __device__ __forceinline__ u32x2 load_half_chunk_fp8_as_bf16(const char *row, in
     return v;
 }
 
+// ---------------------------------------------------------------------------- direct global -> LDS loads
+// A raw buffer descriptor over `bytes` bytes starting at `base`: loads whose byte offset is not
+// below `bytes` return zeros instead of touching memory, which is how tile rows that do not exist
+// (ragged tile edges, rejected picks) are filled.
+typedef __attribute__((address_space(3))) void lds_void_t;
+constexpr uint32_t kVoffInvalid = 0x80000000u;      // never below a descriptor's size (sizes stay under 2 GiB)
+
+__device__ __forceinline__ u32x4 make_rsrc(const void *base, uint32_t bytes)
+{
+    const uint64_t addr = reinterpret_cast<uint64_t>(base);
+    u32x4 r;
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)addr);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(addr >> 32) & 0xffffu);     // stride 0: raw byte offsets
+    r[2] = __builtin_amdgcn_readfirstlane(bytes);
+    r[3] = 0x00020000u;                                                          // 32-bit raw data format
+    return r;
+}
+// One wavefront-wide instruction: lane l fetches the 16 bytes at byte offset voff + soff of the
+// descriptor and the hardware writes them to LDS at `lds_base + 16*l` (lds_base wavefront-uniform),
+// without passing through registers.  Completion is tracked by the vector-memory counter.
+// Written as assembly on purpose: for the builtin form the compiler orders every later LDS read
+// behind all outstanding direct loads, which would serialise the prefetch of the next slab with the
+// reads of the current one.  Callers order the LDS accesses themselves with wait_vmem + a barrier.
+__device__ __forceinline__ void direct_load16(u32x4 rsrc, uint32_t voff, uint32_t soff, char *lds_base)
+{
+    const uint32_t lds_addr = (uint32_t)(uintptr_t)(lds_void_t *)lds_base;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+                 : "memory", "m0");
+}
+// Wait until at most N of this wavefront's vector-memory loads are outstanding (N < 16).
+template <int N> __device__ __forceinline__ void wait_vmem()
+{
+    static_assert(N >= 0 && N < 16, "immediate range");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | N);
+}
+// LDS transpose read: the 16 lanes of a group each point at 4 consecutive 16-bit elements of a
+// row (lanes 4k..4k+3 cover 16 columns of row k, k = 0..3); lane n receives column n of those four
+// rows, i.e. four reduction-consecutive elements of a row-major [reduction][column] tile.
+__device__ __forceinline__ u32x2 lds_read_tr16(const char *at)
+{
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(lds_void_t *)at);
+    return __builtin_bit_cast(u32x2, v);
+}
+
 // ---------------------------------------------------------------------------- LDS tile
 // A tile holds ROWS rows of BK reduction elements, K-major (a row's chunks are adjacent), so
 // an MFMA operand fragment is one 16-byte LDS read per lane.  Chunk positions inside each

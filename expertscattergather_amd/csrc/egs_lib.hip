@@ -9,7 +9,9 @@
 #include "../../include/egs_hip.h"
 #include "egs_device.h"
 #include "egs_rows_gemm.h"
+#include "egs_rows_gemm_dl.h"
 #include "egs_dw.h"
+#include "egs_dw_dl.h"
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
 
@@ -100,6 +102,8 @@ struct DwPlan {
     int BI, BJ, BK, i_tiles, j_tiles, S, rows_per_split;   // general tiled kernel
     bool small_ok;                                          // shape admits the small-expert kernel
     int s_i_tiles, s_j_tiles, s_S, s_rows_per_split;        // its plan
+    bool big_ok;                                            // shape admits the direct-to-LDS kernel (256 x BQ tiles)
+    int b_bq, b_i_tiles, b_j_tiles, b_S, b_rows_per_split;  // its plan
     size_t bytes;                                           // workspace covering whichever runs
 };
 
@@ -124,6 +128,26 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
     pl.S = (int)S;
     pl.rows_per_split = (int)rows;
     pl.bytes = S > 1 ? align_up((size_t)S * d->E * d->I * d->J * 4, 256) : 0;
+
+    // large 16-bit shapes: 256 x 256 (or 256 x 128) tiles, 64-row slabs, splits only to fill the device twice
+    pl.big_ok = act_dtype != EGS_F32 && d->I % 8 == 0 && d->J % 8 == 0 && d->I > 128 && d->J > 64 && Me >= 256 && d->E > 0;
+    if (pl.big_ok) {
+        pl.b_bq = d->J > 128 ? 256 : 128;
+        pl.b_i_tiles = ceil_div(d->I, 256);
+        pl.b_j_tiles = ceil_div(d->J, pl.b_bq);
+        const int64_t tiles = (int64_t)d->E * pl.b_i_tiles * pl.b_j_tiles;
+        int64_t s3 = (512 + tiles - 1) / tiles;
+        const int64_t most = (Me + 255) / 256;              // at least four slabs per split
+        if (s3 > most) s3 = most;
+        if (s3 > 32) s3 = 32;
+        if (s3 < 1) s3 = 1;
+        int64_t r3 = ((Me + s3 - 1) / s3 + 63) / 64 * 64;
+        s3 = (Me + r3 - 1) / r3;
+        pl.b_S = (int)s3;
+        pl.b_rows_per_split = (int)r3;
+        const size_t b3 = s3 > 1 ? align_up((size_t)s3 * d->E * d->I * d->J * 4, 256) : 0;
+        if (b3 > pl.bytes) pl.bytes = b3;
+    }
 
     // small experts: 64 x 64 tiles, up to 1024 picks per workgroup, enough workgroups to cover the device
     pl.small_ok = act_dtype != EGS_F32 && d->I % 8 == 0 && d->J % 8 == 0 && d->I >= 8 && d->J >= 8 && d->I <= 128 &&
@@ -170,6 +194,17 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
             p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
             int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
             if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+            // well-formed shapes take the direct-to-LDS pipeline
+            const bool dl = WES == 2 && !g_force_generic && p.R % kDlBK == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
+                            p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && p.w_scale == nullptr &&
+                            (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
+            if constexpr (WES == 2) {
+                if (dl) {
+                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);
+                    EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
+                    return EGS_OK;
+                }
+            }
             hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 4, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
                                dim3(512), 0, s, p);
         }
@@ -488,6 +523,11 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
     const int64_t w_row = w_trans ? d->J : d->I;
     p.w_vec = WES == 1 ? (aligned_to(W, 8) && w_row % 8 == 0) : (aligned_to(W, 16) && (w_row * WES) % 16 == 0);   // stricter than the 8-byte blocks of the transposed loader need
     p.c_vec = aligned_to(Y, 16) && d->J % 4 == 0;
+    {
+        const uint64_t span = d->B > 0 && d->T > 0
+            ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES : 0;
+        p.a_bytes = span < (1ull << 31) ? (uint32_t)span : 0;
+    }
     if (w_dtype == EGS_FP8_E4M3) {
         return w_trans ? launch_rows_gemm_cfg<ElemBF16, 1, true, true, EPI_STORE>(p, s)
                        : launch_rows_gemm_cfg<ElemBF16, 1, true, false, EPI_STORE>(p, s);
@@ -518,6 +558,10 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     p.a_vec = aligned_to(Y, 16) && ((int64_t)d->J * ES) % 16 == 0;
     const int64_t w_row = w_trans ? d->I : d->J;
     p.w_vec = aligned_to(W, 16) && (w_row * ES) % 16 == 0;
+    {
+        const uint64_t span = (uint64_t)d->B * d->E * d->K * d->J * ES;
+        p.a_bytes = span < (1ull << 31) ? (uint32_t)span : 0;
+    }
 
     if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) {
         float *acc32 = (float *)Out;
@@ -578,6 +622,32 @@ int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *
     p.o_vec = aligned_to(dW, 16) && d->J % 4 == 0;
     p.i_tiles = pl.i_tiles; p.j_tiles = pl.j_tiles; p.S = pl.S; p.rows_per_split = pl.rows_per_split;
     p.out_dtype = out_dtype; p.dw_layout = dw_layout;
+    const uint64_t x_span = d->B > 0 && d->T > 0
+        ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES : 0;
+    const uint64_t y_span = (uint64_t)d->B * d->E * d->K * d->J * ES;
+    if (pl.big_ok && !g_force_generic && p.x_vec && p.y_vec && x_span < (1ull << 31) && y_span < (1ull << 31) &&
+        aligned_to(dW, 16)) {
+        DwDlParams q;
+        q.d = p;
+        q.d.i_tiles = pl.b_i_tiles; q.d.j_tiles = pl.b_j_tiles; q.d.S = pl.b_S; q.d.rows_per_split = pl.b_rows_per_split;
+        q.x_bytes = (uint32_t)x_span; q.y_bytes = (uint32_t)y_span;
+        const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.b_i_tiles * pl.b_j_tiles * pl.b_S;
+        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+        if (act_dtype == EGS_F16) {
+            if (pl.b_bq == 256) hipLaunchKernelGGL((dw_dl_kernel<ElemF16, 256>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
+            else hipLaunchKernelGGL((dw_dl_kernel<ElemF16, 128>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
+        } else {
+            if (pl.b_bq == 256) hipLaunchKernelGGL((dw_dl_kernel<ElemBF16, 256>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
+            else hipLaunchKernelGGL((dw_dl_kernel<ElemBF16, 128>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
+        }
+        EGS_CHECK_LAUNCH("dw_dl_kernel");
+        if (pl.b_S > 1) {
+            hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s, (const float *)workspace,
+                               (char *)dW, pl.b_S, d->E, d->I, d->J, out_dtype, dw_layout);
+            EGS_CHECK_LAUNCH("dw_reduce_kernel");
+        }
+        return EGS_OK;
+    }
     const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.i_tiles * pl.j_tiles * pl.S;
     if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
     switch (act_dtype) {

@@ -32,6 +32,7 @@ struct RowsGemmParams {
     int32_t ind_dtype;
     int32_t a_vec, w_vec, c_vec;   // 1 when 16-byte accesses are safe on that tensor
     int32_t m_tiles, n_tiles;
+    uint32_t a_bytes;       // extent of A in bytes when it is below 2 GiB, else 0 (direct-load kernel only)
 };
 
 template <class TT, int WES, int BM, int BN, int BK, int WM, int WN, bool GATHER, bool W_TRANS, int EPI>

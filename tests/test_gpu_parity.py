@@ -28,6 +28,9 @@ SHAPES = [
     (2, 50, 9, 40, 136, 200),     # N > 128: two column tiles; E not a multiple of 8
     (7, 9, 17, 3, 8, 4),
     (2, 300, 4, 130, 260, 96),    # several reduction slabs and row tiles
+    (3, 300, 5, 200, 192, 256),   # large products: 256 x 256 tiles, ragged last row tile, 192 of 256 columns
+    (2, 128, 9, 260, 128, 200),   # large gather with half a 16-column tile at the edge
+    (2, 200, 3, 128, 256, 72),    # large weight gradient without splits, 72 of 128 columns
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
@@ -169,9 +172,12 @@ def test_scatter_output_does_not_depend_on_stale_memory(mode):
         assert_close(o, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].numpy(), T), torch.bfloat16, "stale")
 
 
-def test_out_of_range_picks_contribute_nothing():
-    B, T, E, K, I, J = 2, 20, 3, 6, 32, 16
-    case = make_case(13, B, T, E, K, I, J, torch.float32)
+@pytest.mark.parametrize("shape,dtype", [((2, 20, 3, 6, 32, 16), torch.float32),
+                                         ((2, 300, 3, 260, 192, 256), torch.bfloat16)],     # second: 256 x 256 tile kernels
+                         ids=["small-f32", "large-bf16"])
+def test_out_of_range_picks_contribute_nothing(shape, dtype):
+    B, T, E, K, I, J = shape
+    case = make_case(13, B, T, E, K, I, J, dtype)
     Ind = case["Ind"].clone()
     Ind[0, 0, 0] = T; Ind[1, 2, 3] = -1; Ind[1, 1, 1] = 10 ** 9
     bad = (Ind < 0) | (Ind >= T)
@@ -184,11 +190,11 @@ def test_out_of_range_picks_contribute_nothing():
     safe = Ind.clone(); safe[bad] = 0
     mask = (~bad).numpy()[..., None]
     refY = O.gather_forward(X, Wg, safe.numpy()) * mask
-    assert_close(got["Y"], refY, torch.float32, "Y with bad picks")
-    assert_close(got["out"], O.scatter_forward(Y * mask, Ws, safe.numpy(), T), torch.float32, "out with bad picks")
+    assert_close(got["Y"], refY, dtype, "Y with bad picks")
+    assert_close(got["out"], O.scatter_forward(Y * mask, Ws, safe.numpy(), T), dtype, "out with bad picks")
     dX, dWg = O.gather_backward(X, Wg, safe.numpy(), Y * mask)
-    assert_close(got["dX"], dX, torch.float32, "dX with bad picks")
-    assert_close(got["dWg"], dWg, torch.float32, "dWg with bad picks")
+    assert_close(got["dX"], dX, dtype, "dX with bad picks")
+    assert_close(got["dWg"], dWg, dtype, "dWg with bad picks")
 
 
 def test_strided_source_rows():
