@@ -72,7 +72,7 @@ int grid_1d(size_t items, int cap = 8192)
 
 // ------------------------------------------------------------------------------ plans
 struct ScatterPlan {
-    size_t seg_off_at, perm_at, rank_at, cnt_at, rows_at;   // byte offsets inside the workspace
+    size_t seg_off_at, perm_at, rank_at, cnt_at, long_tab_at, long_part_at, rows_at;   // byte offsets inside the workspace
     size_t bytes;
 };
 
@@ -85,7 +85,8 @@ struct ScatterPlan {
 // The rows region is always sized for fp32.
 ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
 {
-    ScatterPlan pl = {0, 0, 0, 0, 0, 0};
+    ScatterPlan pl;
+    memset(&pl, 0, sizeof(pl));
     const size_t N = (size_t)d->E * d->K;
     if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) return pl;
     size_t at = 0;
@@ -93,6 +94,9 @@ ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
     pl.perm_at = at;    at += align_up((size_t)d->B * N * 4, 256);
     pl.rank_at = at;    at += align_up((size_t)d->B * N * 4, 256);
     pl.cnt_at = at;     at += d->T > kCsrLdsTokens ? align_up((size_t)d->B * d->T * 4, 256) : 0;
+    // long segments (tokens picked more than kLongSegment times): records and fp32 partial rows
+    pl.long_tab_at = at;  at += align_up((size_t)d->B * long_tab_stride((int)N) * 4, 256);
+    pl.long_part_at = at; at += align_up((size_t)d->B * long_max_slots((int)N) * d->I * 4, 256);
     pl.rows_at = at;    at += align_up((size_t)d->B * N * d->I * 4, 256);
     pl.bytes = at;
     return pl;
@@ -299,7 +303,7 @@ bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, c
 // workgroups of the same launch
 bool make_scatter_rows_small(const void *Y, const void *W, void *rows, bool rows_f32, const egs_dims *d, int act_dtype,
                              int w_layout, bool ride, const void *Ind, int ind_dtype, int32_t *seg_off, int32_t *perm,
-                             int32_t *rank_tmp, SmallRowsJob &j)
+                             int32_t *rank_tmp, int32_t *long_tab, SmallRowsJob &j)
 {
     const int R = d->J, N = d->I;
     if (g_force_generic || !small_shape_ok(act_dtype, R, N)) return false;
@@ -315,7 +319,7 @@ bool make_scatter_rows_small(const void *Y, const void *W, void *rows, bool rows
     p.tiles_per_e = (int)((Me + 255) / 256);
     if (ride) {
         p.csr_blocks = d->B; p.Ind = Ind; p.ind_dtype = ind_dtype;
-        p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp;
+        p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp; p.long_tab = long_tab;
         j.lds = csr_count_lds(d->T, 4);
     }
     if ((int64_t)8 * ceil_div(d->E, 8) * p.tiles_per_e + p.csr_blocks > INT32_MAX / 2) return false;
@@ -418,12 +422,12 @@ int launch_dw_reduce4(const SmallDwJob &j, hipStream_t s)
 // per-wavefront histograms when they fit in LDS, bitonic sort in LDS for long sequences, else
 // the one-wavefront counting sort
 int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int32_t *seg_off, int32_t *perm,
-                         int32_t *rank_tmp, int32_t *cnt, hipStream_t s)
+                         int32_t *rank_tmp, int32_t *cnt, int32_t *long_tab, hipStream_t s)
 {
     const int64_t N = (int64_t)d->E * d->K;
     if (N >= 1) {
-        // as many wavefronts as the per-wavefront histograms leave room for (up to 144 KB of LDS)
-        const size_t budget = 144 * 1024;
+        // as many wavefronts as the per-wavefront histograms leave room for (up to 148 KB of LDS)
+        const size_t budget = 148 * 1024;
         int nw = (int)((N + 63) / 64);
         if (nw > 16) nw = 16;
         while (nw > 1 && csr_count_lds(d->T, nw) > budget) nw >>= 1;
@@ -435,7 +439,7 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
                 if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(csr_count_kernel)");
                 configured = lds;
             }
-            hipLaunchKernelGGL(csr_count_kernel, dim3(d->B), dim3(64 * nw), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, rank_tmp);
+            hipLaunchKernelGGL(csr_count_kernel, dim3(d->B), dim3(64 * nw), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, rank_tmp, long_tab);
             EGS_CHECK_LAUNCH("csr_count_kernel");
             return EGS_OK;
         }
@@ -454,20 +458,20 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
         int threads = NP / 2;
         if (threads < 64) threads = 64;
         if (threads > 1024) threads = 1024;
-        hipLaunchKernelGGL(csr_sort_kernel, dim3(d->B), dim3(threads), lds, s, Ind, ind_dtype, d->T, (int32_t)N, NP, QB, seg_off, perm);
+        hipLaunchKernelGGL(csr_sort_kernel, dim3(d->B), dim3(threads), lds, s, Ind, ind_dtype, d->T, (int32_t)N, NP, QB, seg_off, perm, long_tab);
         EGS_CHECK_LAUNCH("csr_sort_kernel");
         return EGS_OK;
     }
     const size_t lds = d->T > kCsrLdsTokens ? 0 : (size_t)d->T * 4;
-    hipLaunchKernelGGL(csr_build_kernel, dim3(d->B), dim3(kWave), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, cnt);
+    hipLaunchKernelGGL(csr_build_kernel, dim3(d->B), dim3(kWave), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, cnt, long_tab);
     EGS_CHECK_LAUNCH("csr_build_kernel");
     return EGS_OK;
 }
 
 // fixed-order reduction of the product rows per token; when `reduce` is given (and qualifies) the
 // second pass of that weight gradient shares the launch
-int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, const int32_t *perm, void *Out,
-                       const egs_dims *d, int act_dtype, SmallDwJob *reduce, hipStream_t s)
+int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, const int32_t *perm, int32_t *long_tab,
+                       float *long_part, void *Out, const egs_dims *d, int act_dtype, SmallDwJob *reduce, hipStream_t s)
 {
     const int N = d->E * d->K;
     const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
@@ -480,7 +484,10 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
     sp.gx = ceil_div(d->T, kThreads >> sp.tpr_log2);
     sp.gy = d->B;
     while ((int64_t)sp.gx * sp.gy > (1 << 22)) sp.gy = (sp.gy + 1) / 2;     // stride loop over batch elements beyond that
-    const int seg_blocks = sp.gx * sp.gy;
+    sp.long_tab = long_tab; sp.long_part = long_part;
+    const int64_t all_seg_blocks = (int64_t)sp.gx * sp.gy + (int64_t)d->B * long_max_slots(N);
+    if (all_seg_blocks > INT32_MAX / 2) return EGS_ERR_BAD_SHAPE;
+    const int seg_blocks = (int)all_seg_blocks;
     const bool fuse = reduce != nullptr && reduce->done && reduce->q.S > 1 && vw4;
     const int red_blocks = fuse ? grid_1d(reduce->w_elems / 4, 1024) : 0;
 #define EGS_SEGSUM(TT, PT)                                                                                                  \
@@ -579,6 +586,8 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     int32_t *perm = (int32_t *)(ws + pl.perm_at);
     int32_t *rank_tmp = (int32_t *)(ws + pl.rank_at);
     int32_t *cnt = d->T > kCsrLdsTokens ? (int32_t *)(ws + pl.cnt_at) : nullptr;
+    int32_t *long_tab = (int32_t *)(ws + pl.long_tab_at);
+    float *long_part = (float *)(ws + pl.long_part_at);
     void *rows = ws + pl.rows_at;
     bool rows_f32 = (mode == EGS_SCATTER_DETERMINISTIC);
     // small experts: the sort rides along with the product when its histograms are small
@@ -586,14 +595,14 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     SmallRowsJob j;
     int rc;
     if (N > 0 && make_scatter_rows_small(Y, W, rows, rows_f32, d, act_dtype, w_layout, ride, Ind, ind_dtype, seg_off, perm,
-                                         rank_tmp, j)) {
+                                         rank_tmp, long_tab, j)) {
         if (!ride) {
-            rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
+            rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
             if (rc != EGS_OK) return rc;
         }
         rc = launch_rows_small_job(j, dw, s);
     } else {
-        rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, s);
+        rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
         if (rc != EGS_OK) return rc;
         rows_f32 = true;                    // the general kernel writes fp32 rows
         p.C = (char *)rows;
@@ -601,7 +610,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
     }
     if (rc != EGS_OK) return rc;
-    return launch_segment_sum(rows, rows_f32, seg_off, perm, Out, d, act_dtype, dw, s);
+    return launch_segment_sum(rows, rows_f32, seg_off, perm, long_tab, long_part, Out, d, act_dtype, dw, s);
 }
 
 int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,

@@ -14,6 +14,48 @@ constexpr int kCsrLdsTokens = 16384;     // token counters kept in LDS up to thi
 __device__ __forceinline__ int32_t cnt_load(int32_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void cnt_store(int32_t *p, int32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
+// ---------------------------------------------------------------------------- long segments
+// A token picked more than kLongSegment times (hot tokens under skewed routing) is not reduced by
+// the thread group that owns its output row: its segment is cut into chunks of kLongSegment
+// picks, every chunk is summed by a workgroup of its own into an fp32 partial row, and whichever
+// of those workgroups finishes last adds the partial rows in chunk order and writes the output
+// row.  Chunk boundaries and the order of the final additions depend only on the routing table,
+// so the result is still bitwise reproducible.
+//
+// The routing-table kernels leave, per batch element, a table of these tokens:
+//   tab[0]            number of records
+//   tab[4 + 4 r ...]  record r = { token, chunks, first partial-row slot, arrival counter }
+// Records and slots are handed out in whatever order the threads get there; nothing downstream
+// depends on that order.
+constexpr int kLongSegment = 128;
+__host__ __device__ inline int long_max_records(int N) { return N / kLongSegment + 1; }
+__host__ __device__ inline int long_max_slots(int N) { return 2 * (N / kLongSegment) + 2; }
+__host__ __device__ inline size_t long_tab_stride(int N) { return 4 + 4 * (size_t)long_max_records(N); }
+
+// Called by every thread of the workgroup that built batch element b's segment offsets, after
+// those are final in global memory (`seg_off_b` = that element's T+1 offsets).
+__device__ __forceinline__ void emit_long_tokens(const int32_t *seg_off_b, int T, int N, int32_t *long_tab, int b, int tid,
+                                                 int nthreads)
+{
+    __shared__ int32_t long_ctr[2];
+    if (long_tab == nullptr) return;
+    int32_t *tab = long_tab + (size_t)b * long_tab_stride(N);
+    if (tid == 0) { long_ctr[0] = 0; long_ctr[1] = 0; }
+    __syncthreads();            // also orders the seg_off stores of the other threads before the loads below
+    for (int t = tid; t < T; t += nthreads) {
+        const int len = seg_off_b[t + 1] - seg_off_b[t];
+        if (len > kLongSegment) {
+            const int nch = (len + kLongSegment - 1) / kLongSegment;
+            const int r = atomicAdd(&long_ctr[0], 1);
+            const int slot = atomicAdd(&long_ctr[1], nch);
+            int32_t *rec = tab + 4 + 4 * r;
+            rec[0] = t; rec[1] = nch; rec[2] = slot; rec[3] = 0;
+        }
+    }
+    __syncthreads();
+    if (tid == 0) tab[0] = long_ctr[0];
+}
+
 __device__ __forceinline__ int wave_inclusive_scan(int v, int lane)
 {
 #pragma unroll
@@ -34,7 +76,8 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane)
 // 64-pick chunk come from ballots over the bits of the token id, not from atomics, so the
 // result does not depend on hardware ordering.  Works for any T and N; slow for large N.
 __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
-                                                          int32_t *seg_off, int32_t *perm, int32_t *cnt_global)
+                                                          int32_t *seg_off, int32_t *perm, int32_t *cnt_global,
+                                                          int32_t *long_tab)
 {
     extern __shared__ int32_t cnt_lds[];
     const int lane = (int)threadIdx.x, b = (int)blockIdx.x;
@@ -84,6 +127,7 @@ __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32
         }
         __syncthreads();                             // cursor update visible to the next chunk
     }
+    emit_long_tokens(seg_off + (size_t)b * (T + 1), T, N, long_tab, b, lane, kWave);
 }
 
 // Fast version when T counters per wavefront fit in LDS: one workgroup of NW wavefronts per
@@ -94,7 +138,7 @@ __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32
 // LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch.
 __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, int nthreads, const void *Ind,
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
-                                               int32_t *perm, int32_t *rank_tmp)
+                                               int32_t *perm, int32_t *rank_tmp, int32_t *long_tab)
 {
     constexpr int MAXC = 8;                             // 64-pick chunks whose tokens (and ranks) are held in registers at a time
     const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
@@ -216,14 +260,16 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
                 if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rr[c]] = q0 + c * kWave + lane;
         }
     }
+    emit_long_tokens(tok_start, T, N, long_tab, b, tid, nthreads);
 }
 
 __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
-                                                         int32_t *seg_off, int32_t *perm, int32_t *rank_tmp)
+                                                         int32_t *seg_off, int32_t *perm, int32_t *rank_tmp,
+                                                         int32_t *long_tab)
 {
     extern __shared__ int32_t sh_cnt_dyn[];
     csr_count_body(sh_cnt_dyn, (int)blockIdx.x, (int)threadIdx.x, (int)blockDim.x, Ind, ind_dtype, T, N, seg_off, perm,
-                   rank_tmp);
+                   rank_tmp, long_tab);
 }
 
 // Fast version for N <= 32768 picks whose (token, pick) pair fits 32 bits: one workgroup per
@@ -231,7 +277,8 @@ __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_
 // unique, so the sorted order is the stable order by token.  NP = N rounded up to a power of
 // two; dynamic LDS = NP * 4 bytes.
 __global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
-                                                        int32_t NP, int32_t QB, int32_t *seg_off, int32_t *perm)
+                                                        int32_t NP, int32_t QB, int32_t *seg_off, int32_t *perm,
+                                                        int32_t *long_tab)
 {
     extern __shared__ uint32_t keys[];
     const int tid = (int)threadIdx.x, nthreads = (int)blockDim.x, b = (int)blockIdx.x;
@@ -273,6 +320,7 @@ __global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t
         }
         seg_off[(size_t)b * (T + 1) + t] = lo;
     }
+    emit_long_tokens(seg_off + (size_t)b * (T + 1), T, N, long_tab, b, tid, nthreads);
 }
 
 // out[b,t,:] = sum, in routing-table order, of the product rows of the picks of token t
@@ -286,6 +334,8 @@ struct SegSumParams {
     int32_t B, T, N, I;
     int32_t tpr_log2;           // 2^tpr_log2 threads share an output row
     int32_t gx, gy;             // logical grid: gx row groups x gy batch slots
+    int32_t *long_tab;          // long-segment records (see emit_long_tokens), or nullptr
+    float *long_part;           // [B, long_max_slots(N), I] fp32 partial rows
 };
 
 template <class TT, class PT, int VW>
@@ -305,6 +355,7 @@ __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const i
     for (int iv = (int)threadIdx.x & (tpr - 1); iv < IV; iv += tpr) {
         const size_t row = (size_t)b * T + t;
         int s0 = seg_off[(size_t)b * (T + 1) + t], s1 = seg_off[(size_t)b * (T + 1) + t + 1];
+        if (sp.long_tab != nullptr && s1 - s0 > kLongSegment) continue;      // segment_sum_long_body writes this row
         float acc[VW];
 #pragma unroll
         for (int x = 0; x < VW; ++x) acc[x] = 0.f;
@@ -395,10 +446,122 @@ __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const i
     }
 }
 
+// One chunk of a long segment: workgroup (b, slot) sums the up to kLongSegment product rows of its
+// chunk into partial row `slot`; the workgroup that arrives last at the record's counter adds the
+// token's partial rows in chunk order and writes the output row.  Slots no record covers exit.
+template <class TT, class PT, int VW>
+__device__ __forceinline__ void segment_sum_long_body(const SegSumParams &sp, const int b, const int slot)
+{
+    __shared__ int32_t sh_rec, sh_last;
+    const int tid = (int)threadIdx.x;
+    const int T = sp.T, N = sp.N, I = sp.I;
+    int32_t *tab = sp.long_tab + (size_t)b * long_tab_stride(N);
+    const int nrec = tab[0];
+    if (nrec == 0) return;
+    if (tid == 0) sh_rec = -1;
+    __syncthreads();
+    for (int r = tid; r < nrec; r += kThreads) {
+        const int first = tab[4 + 4 * r + 2], nch = tab[4 + 4 * r + 1];
+        if (slot >= first && slot < first + nch) sh_rec = r;
+    }
+    __syncthreads();
+    const int r = sh_rec;
+    if (r < 0) return;
+    int32_t *rec = tab + 4 + 4 * r;
+    const int t = rec[0], nch = rec[1], first = rec[2];
+    const int c = slot - first;
+    const int seg0 = sp.seg_off[(size_t)b * (T + 1) + t], seg1 = sp.seg_off[(size_t)b * (T + 1) + t + 1];
+    const int s0 = seg0 + c * kLongSegment, s1 = min(seg1, s0 + kLongSegment);
+    const int IV = (I + VW - 1) / VW;
+    const PT *P = reinterpret_cast<const PT *>(sp.P);
+    const int32_t *pb = sp.perm + (size_t)b * N;
+    const size_t slots = (size_t)long_max_slots(N);
+    float *part = sp.long_part + ((size_t)b * slots + slot) * I;
+
+    for (int iv = tid; iv < IV; iv += kThreads) {
+        const PT *Pb = P + (size_t)b * N * I + (size_t)iv * VW;
+        float acc[VW];
+#pragma unroll
+        for (int x = 0; x < VW; ++x) acc[x] = 0.f;
+        auto add_elems = [&](const PT *src) {
+#pragma unroll
+            for (int x = 0; x < VW; ++x) {
+                if constexpr (sizeof(PT) == 4) acc[x] += src[x];
+                else acc[x] += TT::ID == 2 ? bf16_bits_to_f32((uint32_t)src[x]) : f16_bits_to_f32((uint32_t)src[x]);
+            }
+        };
+        int s = s0;
+        for (; s + 8 <= s1; s += 8) {                    // 8 rows in flight, added in table order
+            int q[8];
+            PT v[8][VW];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) q[u] = pb[s + u];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const PT *src = Pb + (size_t)q[u] * I;
+                if constexpr (VW == 4) {
+                    typedef typename std::conditional<sizeof(PT) == 4, f32x4, u32x2>::type vec_t;
+                    *reinterpret_cast<vec_t *>(v[u]) = *reinterpret_cast<const vec_t *>(src);
+                } else {
+                    v[u][0] = src[0];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) add_elems(v[u]);
+        }
+        for (; s < s1; ++s) {
+            const PT *src = Pb + (size_t)pb[s] * I;
+            PT v[VW];
+#pragma unroll
+            for (int x = 0; x < VW; ++x) v[x] = src[x];
+            add_elems(v);
+        }
+#pragma unroll
+        for (int x = 0; x < VW; ++x) part[(size_t)iv * VW + x] = acc[x];
+    }
+    __threadfence();                    // partial row visible device-wide before the arrival is counted
+    __syncthreads();
+    if (tid == 0) sh_last = (atomicAdd(&rec[3], 1) == nch - 1) ? 1 : 0;
+    __syncthreads();
+    if (!sh_last) return;
+    __threadfence();                    // see the partial rows of the workgroups that arrived earlier
+    const float *pt = sp.long_part + ((size_t)b * slots + first) * I;
+    for (int iv = tid; iv < IV; iv += kThreads) {
+        float acc[VW];
+#pragma unroll
+        for (int x = 0; x < VW; ++x) acc[x] = 0.f;
+        for (int cc = 0; cc < nch; ++cc) {
+#pragma unroll
+            for (int x = 0; x < VW; ++x)
+                acc[x] += __builtin_nontemporal_load(pt + (size_t)cc * I + (size_t)iv * VW + x);
+        }
+        const size_t at = ((size_t)b * T + t) * I + (size_t)iv * VW;
+#pragma unroll
+        for (int x = 0; x < VW; ++x) {
+            if constexpr (TT::ES == 4) reinterpret_cast<float *>(sp.out)[at + x] = acc[x];
+            else reinterpret_cast<uint16_t *>(sp.out)[at + x] = (uint16_t)f32_to_elem_bits<TT>(acc[x]);
+        }
+    }
+}
+
+// workgroups [0, gx*gy): ordinary rows; then B * long_max_slots(N) workgroups for long segments
+template <class TT, class PT, int VW>
+__device__ __forceinline__ void segment_sum_dispatch(const SegSumParams &sp, const int block)
+{
+    const int seg_blocks = sp.gx * sp.gy;
+    if (block < seg_blocks) {
+        segment_sum_body<TT, PT, VW>(sp, block % sp.gx, block / sp.gx);
+    } else {
+        const int slots = long_max_slots(sp.N);
+        const int lb = block - seg_blocks;
+        segment_sum_long_body<TT, PT, VW>(sp, lb / slots, lb % slots);
+    }
+}
+
 template <class TT, class PT, int VW>
 __global__ __launch_bounds__(kThreads) void segment_sum_kernel(SegSumParams sp)
 {
-    segment_sum_body<TT, PT, VW>(sp, (int)blockIdx.x % sp.gx, (int)blockIdx.x / sp.gx);
+    segment_sum_dispatch<TT, PT, VW>(sp, (int)blockIdx.x);
 }
 
 // zero n floats (the atomic mode's accumulator).  A kernel rather than a memset so that the

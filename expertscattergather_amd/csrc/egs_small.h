@@ -40,7 +40,7 @@ struct SmallRowsParams {
     int32_t rows_share_xcd; // 1: row tiles map to XCDs (source rows reused across experts), 0: experts map to XCDs
     // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
     int32_t csr_blocks;
-    int32_t *seg_off, *perm, *rank_tmp;
+    int32_t *seg_off, *perm, *rank_tmp, *long_tab;
     unsigned long long *dbg_times;   // optional [grid*4][2] wall-clock stamps per wavefront (performance debugging)
 };
 
@@ -56,7 +56,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     if constexpr (!GATHER) {
         if (block < p.csr_blocks) {
             csr_count_body(sh_cnt_small, block, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
-                           p.E * p.K, p.seg_off, p.perm, p.rank_tmp);
+                           p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
             return;
         }
     }
@@ -442,13 +442,13 @@ __global__ __launch_bounds__(kThreads) void rows_dw_small_kernel(SmallRowsParams
 }
 
 // segment sums of a scatter and the second pass of a weight gradient in one launch:
-// workgroups [0, seg_blocks) reduce product rows per token, the rest sum dW partials
+// workgroups [0, seg_blocks) reduce product rows per token (ordinary and long segments), the rest sum dW partials
 template <class TT, class PT, int VW>
 __global__ __launch_bounds__(kThreads) void segsum_dwreduce_kernel(SegSumParams sp, int seg_blocks, const float *part,
                                                                    char *dW, int32_t S, size_t total4, int32_t out_dtype)
 {
     const int block = (int)blockIdx.x;
-    if (block < seg_blocks) segment_sum_body<TT, PT, VW>(sp, block % sp.gx, block / sp.gx);
+    if (block < seg_blocks) segment_sum_dispatch<TT, PT, VW>(sp, block);
     else dw_reduce4_body(part, dW, S, total4, out_dtype, block - seg_blocks, (int)gridDim.x - seg_blocks);
 }
 

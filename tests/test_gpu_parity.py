@@ -151,6 +151,45 @@ def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
     del junk
 
 
+@pytest.mark.parametrize("shape,dtype", [((3, 40, 6, 100, 24, 16), torch.float32),      # small-expert rows, table built by the general sorter
+                                         ((2, 64, 8, 64, 128, 64), torch.bfloat16),     # small-expert rows, table rides along
+                                         ((2, 50, 4, 300, 30, 24), torch.float16),      # I not a multiple of 4: scalar columns
+                                         ((2, 300, 4, 200, 256, 192), torch.bfloat16)], # 256 x 256 tile rows
+                         ids=lambda v: "x".join(map(str, v)) if isinstance(v, tuple) else str(v).split(".")[-1])
+@pytest.mark.parametrize("mode", ["deterministic", "atomic"])
+def test_long_segments_are_reduced_in_chunks(shape, dtype, mode):
+    # tokens picked far more often than one thread group reduces in one go: segment lengths around the
+    # chunk size (127, 128, 129), several chunks (300+), one token taking most picks, and empty tokens
+    B, T, E, K, I, J = shape
+    case = make_case(21, B, T, E, K, I, J, dtype)
+    N = E * K
+    gen = torch.Generator().manual_seed(5)
+    Ind = torch.empty(B, N, dtype=torch.int64)
+    for b in range(B):
+        lens = [127, 128, 129] if b == 0 else [N // 2 + 3, 257]
+        lens = [n for n in lens if n > 0]
+        while sum(lens) > N:
+            lens.pop()
+        toks = torch.randperm(T, generator=gen)
+        flat = torch.cat([torch.full((n,), int(toks[i])) for i, n in enumerate(lens)] +
+                         [toks[len(lens) + torch.randint(0, max(1, T // 2 - len(lens)), (N - sum(lens),), generator=gen)]])
+        Ind[b] = flat[torch.randperm(N, generator=gen)]
+    Ind = Ind.reshape(B, E, K)
+    hk.set_scatter_mode(mode)
+    Y, Ws = dev(case["Y"]), dev(case["Ws"])
+    got = hk.expert_scatter_forward_call(Y, Ws, dev(Ind), T, torch.float32)
+    ref = O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), Ind.numpy(), T)
+    hk.set_scatter_mode("deterministic")
+    assert_close(got, ref, dtype, "long segments")
+    if mode == "deterministic":
+        hk.set_scatter_mode(mode)
+        for _ in range(3):
+            assert torch.equal(got, hk.expert_scatter_forward_call(Y, Ws, dev(Ind), T, torch.float32))
+    # the same table drives dX
+    dX = hk.expert_gather_backward_call(dev(case["X"]), dev(case["Wg"]), dev(Ind), Y, torch.float32)[0]
+    assert_close(dX, O.gather_backward(np64(case["X"]), np64(case["Wg"]), Ind.numpy(), np64(case["Y"]))[0], dtype, "dX long segments")
+
+
 @pytest.mark.parametrize("mode", ["deterministic", "atomic"])
 def test_scatter_output_does_not_depend_on_stale_memory(mode):
     # the reference allocates the scatter output with torch.empty and only adds into it
