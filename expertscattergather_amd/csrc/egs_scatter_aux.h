@@ -22,12 +22,17 @@ __device__ __forceinline__ void cnt_store(int32_t *p, int32_t v) { __hip_atomic_
 // row.  Chunk boundaries and the order of the final additions depend only on the routing table,
 // so the result is still bitwise reproducible.
 //
+// Partial rows cross workgroups (and L2s) inside one kernel.  They are written and read with
+// device-scope atomic accesses, which go through to memory, and a workgroup counts its arrival
+// only after its stores have completed; a device-scope fence would do as well, but it writes back
+// and invalidates the whole L2 each time, which on skewed routing cost more than the reduction.
+//
 // The routing-table kernels leave, per batch element, a table of these tokens:
 //   tab[0]            number of records
 //   tab[4 + 4 r ...]  record r = { token, chunks, first partial-row slot, arrival counter }
 // Records and slots are handed out in whatever order the threads get there; nothing downstream
 // depends on that order.
-constexpr int kLongSegment = 128;
+constexpr int kLongSegment = 64;
 __host__ __device__ inline int long_max_records(int N) { return N / kLongSegment + 1; }
 __host__ __device__ inline int long_max_slots(int N) { return 2 * (N / kLongSegment) + 2; }
 __host__ __device__ inline size_t long_tab_stride(int N) { return 4 + 4 * (size_t)long_max_records(N); }
@@ -516,45 +521,69 @@ __device__ __forceinline__ void segment_sum_long_body(const SegSumParams &sp, co
             for (int x = 0; x < VW; ++x) v[x] = src[x];
             add_elems(v);
         }
-#pragma unroll
-        for (int x = 0; x < VW; ++x) part[(size_t)iv * VW + x] = acc[x];
+        if constexpr (VW == 4) {
+            uint64_t *dst = reinterpret_cast<uint64_t *>(part + (size_t)iv * 4);
+            __hip_atomic_store(dst, (uint64_t)f32_bits(acc[0]) | ((uint64_t)f32_bits(acc[1]) << 32), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(dst + 1, (uint64_t)f32_bits(acc[2]) | ((uint64_t)f32_bits(acc[3]) << 32), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+            __hip_atomic_store(part + iv, acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    __threadfence();                    // partial row visible device-wide before the arrival is counted
-    __syncthreads();
-    if (tid == 0) sh_last = (atomicAdd(&rec[3], 1) == nch - 1) ? 1 : 0;
+    __builtin_amdgcn_s_waitcnt(0);      // this thread's partial-row stores have completed
+    __syncthreads();                    // ... and so have everybody else's, before the arrival is counted
+    if (tid == 0)
+        sh_last = (__hip_atomic_fetch_add(&rec[3], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nch - 1) ? 1 : 0;
     __syncthreads();
     if (!sh_last) return;
-    __threadfence();                    // see the partial rows of the workgroups that arrived earlier
     const float *pt = sp.long_part + ((size_t)b * slots + first) * I;
     for (int iv = tid; iv < IV; iv += kThreads) {
         float acc[VW];
 #pragma unroll
         for (int x = 0; x < VW; ++x) acc[x] = 0.f;
         for (int cc = 0; cc < nch; ++cc) {
-#pragma unroll
-            for (int x = 0; x < VW; ++x)
-                acc[x] += __builtin_nontemporal_load(pt + (size_t)cc * I + (size_t)iv * VW + x);
+            const float *src = pt + (size_t)cc * I + (size_t)iv * VW;
+            if constexpr (VW == 4) {
+                const uint64_t lo = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const uint64_t hi = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                acc[0] += bits_f32((uint32_t)lo); acc[1] += bits_f32((uint32_t)(lo >> 32));
+                acc[2] += bits_f32((uint32_t)hi); acc[3] += bits_f32((uint32_t)(hi >> 32));
+            } else {
+                acc[0] += __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
         const size_t at = ((size_t)b * T + t) * I + (size_t)iv * VW;
-#pragma unroll
-        for (int x = 0; x < VW; ++x) {
-            if constexpr (TT::ES == 4) reinterpret_cast<float *>(sp.out)[at + x] = acc[x];
-            else reinterpret_cast<uint16_t *>(sp.out)[at + x] = (uint16_t)f32_to_elem_bits<TT>(acc[x]);
+        if constexpr (TT::ES == 4) {
+            float *dst = reinterpret_cast<float *>(sp.out) + at;
+            if constexpr (VW == 4) *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+            else dst[0] = acc[0];
+        } else {
+            uint16_t *dst = reinterpret_cast<uint16_t *>(sp.out) + at;
+            if constexpr (VW == 4) {
+                u32x2 w;
+                w[0] = pack2<TT>(acc[0], acc[1]);
+                w[1] = pack2<TT>(acc[2], acc[3]);
+                *reinterpret_cast<u32x2 *>(dst) = w;
+            } else {
+                dst[0] = (uint16_t)f32_to_elem_bits<TT>(acc[0]);
+            }
         }
     }
 }
 
-// workgroups [0, gx*gy): ordinary rows; then B * long_max_slots(N) workgroups for long segments
+// workgroups [0, B * long_max_slots(N)): chunks of long segments (first, because they are the longest
+// dependent chains of the launch); then gx * gy workgroups for the ordinary rows
 template <class TT, class PT, int VW>
 __device__ __forceinline__ void segment_sum_dispatch(const SegSumParams &sp, const int block)
 {
-    const int seg_blocks = sp.gx * sp.gy;
-    if (block < seg_blocks) {
-        segment_sum_body<TT, PT, VW>(sp, block % sp.gx, block / sp.gx);
+    const int slots = long_max_slots(sp.N);
+    const int long_blocks = sp.B * slots;
+    if (block < long_blocks) {
+        segment_sum_long_body<TT, PT, VW>(sp, block / slots, block % slots);
     } else {
-        const int slots = long_max_slots(sp.N);
-        const int lb = block - seg_blocks;
-        segment_sum_long_body<TT, PT, VW>(sp, lb / slots, lb % slots);
+        const int sb = block - long_blocks;
+        segment_sum_body<TT, PT, VW>(sp, sb % sp.gx, sb / sp.gx);
     }
 }
 

@@ -159,14 +159,14 @@ def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
 @pytest.mark.parametrize("mode", ["deterministic", "atomic"])
 def test_long_segments_are_reduced_in_chunks(shape, dtype, mode):
     # tokens picked far more often than one thread group reduces in one go: segment lengths around the
-    # chunk size (127, 128, 129), several chunks (300+), one token taking most picks, and empty tokens
+    # chunk size and its double (63, 64, 65, 127, 128, 129), many chunks, one token taking most picks, and empty tokens
     B, T, E, K, I, J = shape
     case = make_case(21, B, T, E, K, I, J, dtype)
     N = E * K
     gen = torch.Generator().manual_seed(5)
     Ind = torch.empty(B, N, dtype=torch.int64)
     for b in range(B):
-        lens = [127, 128, 129] if b == 0 else [N // 2 + 3, 257]
+        lens = [63, 64, 65, 127, 128, 129] if b == 0 else [N // 2 + 3, 193]
         lens = [n for n in lens if n > 0]
         while sum(lens) > N:
             lens.pop()
