@@ -79,8 +79,8 @@ struct ScatterPlan {
 // Workspace of the GEMM-scatter: routing table (segment offsets, picks in token order, scratch
 // ranks, optional global counters) and the product rows in pick order.
 //   deterministic mode: product rows in fp32 -> fp32 accumulation with one final rounding;
-//   atomic ("fast") mode: with 16-bit element types the small-expert kernel keeps the product
-//   rows in the element type (half the traffic, one extra rounding per pick; the summation
+//   atomic ("fast") mode: with 16-bit element types the product rows are kept in the element
+//   type (half the traffic, one extra rounding per pick; the summation
 //   order is still fixed); fp32 uses global atomics on the output, no workspace.
 // The rows region is always sized for fp32.
 ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
@@ -174,6 +174,9 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
     return pl;
 }
 
+// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
+size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
+
 // ------------------------------------------------------------------------------ rows-GEMM dispatch
 template <class TT, int WES, bool GATHER, bool W_TRANS, int EPI>
 int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
@@ -204,6 +207,9 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                             (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
             if constexpr (WES == 2) {
                 if (dl) {
+                    if (GATHER || csr_count_lds(p.T, kThreads / kWave) > (size_t)2 * kDlStageBytes) p.csr_blocks = 0;
+                    grid += p.csr_blocks;
+                    p.csr_done = p.csr_blocks > 0;
                     hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);
                     EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
                     return EGS_OK;
@@ -244,9 +250,6 @@ int launch_rows_gemm(RowsGemmParams &p, int act_dtype, bool w_trans, hipStream_t
 
 // ------------------------------------------------------------------------------ small-expert fast paths
 constexpr uint64_t kSpan32 = 0xFFFFFFFFull;      // the small kernels address with 32-bit byte offsets
-
-// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
-size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
 
 bool small_shape_ok(int act_dtype, int R, int N)
 {
@@ -602,12 +605,15 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         }
         rc = launch_rows_small_job(j, dw, s);
     } else {
-        rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
-        if (rc != EGS_OK) return rc;
-        rows_f32 = true;                    // the general kernel writes fp32 rows
+        rows_f32 = mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32;   // fast mode: rows in the element type
         p.C = (char *)rows;
         p.c_vec = d->I % 4 == 0;
-        rc = launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s);
+        // the routing table may ride along with the product launch (large shapes); otherwise it is a launch of its own
+        p.csr_blocks = N > 0 ? d->B : 0; p.csr_done = 0;
+        p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp; p.long_tab = long_tab;
+        rc = rows_f32 ? launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s)
+                      : launch_rows_gemm<false, EPI_STORE>(p, act_dtype, w_trans, s);
+        if (rc == EGS_OK && !p.csr_done) rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
     }
     if (rc != EGS_OK) return rc;
     return launch_segment_sum(rows, rows_f32, seg_off, perm, long_tab, long_part, Out, d, act_dtype, dw, s);

@@ -33,6 +33,10 @@ struct RowsGemmParams {
     int32_t a_vec, w_vec, c_vec;   // 1 when 16-byte accesses are safe on that tensor
     int32_t m_tiles, n_tiles;
     uint32_t a_bytes;       // extent of A in bytes when it is below 2 GiB, else 0 (direct-load kernel only)
+    // routing table of the scatter built by the first csr_blocks (= B) workgroups of the product launch
+    // (direct-load kernel only; csr_done reports that the launch took it along)
+    int32_t csr_blocks, csr_done;
+    int32_t *seg_off, *perm, *rank_tmp, *long_tab;
 };
 
 template <class TT, int WES, int BM, int BN, int BK, int WM, int WN, bool GATHER, bool W_TRANS, int EPI>

@@ -19,6 +19,7 @@
 // part of expert_scatter_kernel (:156-247) on these shapes.
 #pragma once
 #include "egs_rows_gemm.h"
+#include "egs_scatter_aux.h"
 
 namespace egs {
 
@@ -47,11 +48,23 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
     __shared__ uint32_t a_voff[BM];
     __shared__ int64_t c_off[BM];
 
+    const int tid = (int)threadIdx.x;
+    int block = (int)blockIdx.x;
+    if constexpr (!GATHER) {
+        // the scatter's routing table does not depend on the product: one workgroup per batch element
+        // builds it here (four wavefronts, histograms in the slab buffers) instead of in a launch of its own
+        if (block < p.csr_blocks) {
+            if (tid >= kThreads) return;
+            csr_count_body(reinterpret_cast<int32_t *>(smem), block, tid, kThreads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
+                           p.seg_off, p.perm, p.rank_tmp, p.long_tab);
+            return;
+        }
+        block -= p.csr_blocks;
+    }
     int e, tile;
-    if (!decode_expert_tile((int)blockIdx.x, p.m_tiles * p.n_tiles, p.E, e, tile)) return;
+    if (!decode_expert_tile(block, p.m_tiles * p.n_tiles, p.E, e, tile)) return;
     const int mt = tile / p.n_tiles, nt = tile - mt * p.n_tiles;
     const int m0 = mt * BM, n0 = nt * BN;
-    const int tid = (int)threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int R = p.R, N = p.N;
