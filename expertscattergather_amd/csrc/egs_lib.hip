@@ -207,7 +207,10 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                             (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
             if constexpr (WES == 2) {
                 if (dl) {
-                    if (GATHER || csr_count_lds(p.T, kThreads / kWave) > (size_t)2 * kDlStageBytes) p.csr_blocks = 0;
+                    p.csr_threads = kDlThreads;         // as many wavefronts as the histograms leave room for
+                    while (p.csr_threads > kWave && csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter)
+                        p.csr_threads >>= 1;
+                    if (GATHER || csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter) p.csr_blocks = 0;
                     grid += p.csr_blocks;
                     p.csr_done = p.csr_blocks > 0;
                     hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);

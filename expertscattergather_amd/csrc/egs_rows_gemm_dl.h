@@ -26,6 +26,8 @@ namespace egs {
 constexpr int kDlBM = 256, kDlBN = 256, kDlBK = 64, kDlThreads = 512;
 constexpr int kDlTileBytes = 256 * 64 * 2;              // one operand slab
 constexpr int kDlStageBytes = 2 * kDlTileBytes;
+constexpr int kDlSmemBytes = 2 * kDlStageBytes + kDlBM * 4 + kDlBM * 8;
+constexpr int kDlSmemBytesScatter = 150 * 1024;
 
 // swizzle of the [reduction][column] tile: 32-byte units of a row are XORed with bits {0,1,3} of
 // the row number, which spreads the 16 rows one transpose read touches over all banks
@@ -44,18 +46,20 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
     constexpr int BM = kDlBM, BN = kDlBN, BK = kDlBK;
     constexpr int TM = 8, TN = 4;                        // 16 x 16 tiles per wavefront: 128 x 64
 
-    __shared__ __attribute__((aligned(1024))) char smem[2 * kDlStageBytes];
-    __shared__ uint32_t a_voff[BM];
-    __shared__ int64_t c_off[BM];
+    // two slab stages, then the row tables; the scatter variants reserve more so that the routing-table
+    // workgroups riding along have room for eight wavefronts' histograms at T = 4096
+    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? kDlSmemBytes : kDlSmemBytesScatter];
+    uint32_t *a_voff = reinterpret_cast<uint32_t *>(smem + 2 * kDlStageBytes);
+    int64_t *c_off = reinterpret_cast<int64_t *>(smem + 2 * kDlStageBytes + BM * 4);
 
     const int tid = (int)threadIdx.x;
     int block = (int)blockIdx.x;
     if constexpr (!GATHER) {
         // the scatter's routing table does not depend on the product: one workgroup per batch element
-        // builds it here (four wavefronts, histograms in the slab buffers) instead of in a launch of its own
+        // builds it here (csr_threads of the workgroup, histograms in the slab buffers) instead of in a launch of its own
         if (block < p.csr_blocks) {
-            if (tid >= kThreads) return;
-            csr_count_body(reinterpret_cast<int32_t *>(smem), block, tid, kThreads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
+            if (tid >= p.csr_threads) return;
+            csr_count_body(reinterpret_cast<int32_t *>(smem), block, tid, p.csr_threads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
                            p.seg_off, p.perm, p.rank_tmp, p.long_tab);
             return;
         }
