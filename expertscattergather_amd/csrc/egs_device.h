@@ -271,6 +271,17 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char *at)
     return __builtin_bit_cast(u32x2, v);
 }
 
+// 8-bit LDS transpose read: of 16 lanes, lanes 2k and 2k+1 point at bytes 0..7 and 8..15 of row k
+// (k = 0..7); lane n receives byte n of those eight rows, i.e. eight reduction-consecutive fp8 values
+// of column n of a row-major [reduction][column] byte tile.
+__device__ __forceinline__ u32x2 lds_read_tr8(const char *at)
+{
+    typedef int i32x2 __attribute__((ext_vector_type(2)));
+    typedef __attribute__((address_space(3))) i32x2 lds_i32x2;
+    i32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_i32x2 *)(lds_void_t *)at);
+    return __builtin_bit_cast(u32x2, v);
+}
+
 // ---------------------------------------------------------------------------- LDS tile
 // A tile holds ROWS rows of BK reduction elements, K-major (a row's chunks are adjacent), so
 // an MFMA operand fragment is one 16-byte LDS read per lane.  Chunk positions inside each

@@ -202,10 +202,11 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
             int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
             if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
             // well-formed shapes take the direct-to-LDS pipeline
-            const bool dl = WES == 2 && !g_force_generic && p.R % kDlBK == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
-                            p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && p.w_scale == nullptr &&
+            const bool dl = !g_force_generic && p.R % kDlBK == 0 && p.N % (WES == 1 ? 16 : 8) == 0 && p.a_vec && p.w_vec &&
+                            p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && (WES == 1 || p.w_scale == nullptr) &&
+                            (WES == 2 || aligned_to(p.W, 16)) &&
                             (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
-            if constexpr (WES == 2) {
+            if constexpr (WES == 2 || W_TRANS) {
                 if (dl) {
                     p.csr_threads = kDlThreads;         // as many wavefronts as the histograms leave room for
                     while (p.csr_threads > kWave && csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter)
@@ -213,7 +214,7 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                     if (GATHER || csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter) p.csr_blocks = 0;
                     grid += p.csr_blocks;
                     p.csr_done = p.csr_blocks > 0;
-                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);
+                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);
                     EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
                     return EGS_OK;
                 }

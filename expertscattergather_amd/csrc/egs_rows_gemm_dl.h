@@ -13,7 +13,10 @@
 //     stays that way in LDS and is read with the transpose read, so no register transposes.
 //
 // Preconditions (checked by the host, which otherwise uses rows_gemm_kernel): 16-bit elements,
-// R % 64 == 0, N % 8 == 0, 16-byte aligned rows, operands below 2 GiB.
+// R % 64 == 0, N % 8 == 0, 16-byte aligned rows, operands below 2 GiB.  fp8 (e4m3) weights in the
+// [reduction][column] layout are supported with bf16 activations (N % 16 == 0): the bytes go to LDS as
+// they are, the 8-bit transpose read hands each lane eight reduction-consecutive values and those are
+// widened to bf16 (exactly) in registers.
 //
 // Replaces the reference's expert_gather_kernel (egs/triton_kernels.py:49-143) and the product
 // part of expert_scatter_kernel (:156-247) on these shapes.
@@ -38,10 +41,12 @@ __device__ __forceinline__ int tr_swizzle(int row) { return (row & 3) | (((row >
 __device__ __forceinline__ int kmajor_key_rows(int row) { return row & 7; }
 __device__ __forceinline__ int kmajor_key_relabelled(int row) { return (((row >> 4) & 3) << 1) | ((row >> 1) & 1); }
 
-template <class TT, bool GATHER, bool W_TRANS, int EPI>
+template <class TT, int WES, bool GATHER, bool W_TRANS, int EPI>
 __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams p)
 {
     static_assert(TT::ES == 2, "16-bit element types");
+    static_assert(WES == 2 || (WES == 1 && W_TRANS && TT::ID == 2), "fp8 weights: [reduction][column] layout, widened to bf16");
+    constexpr bool W_FP8 = (WES == 1);
     static_assert(EPI == EPI_STORE || EPI == EPI_STORE_F32, "plain stores only");
     constexpr int BM = kDlBM, BN = kDlBN, BK = kDlBK;
     constexpr int TM = 8, TN = 4;                        // 16 x 16 tiles per wavefront: 128 x 64
@@ -96,7 +101,7 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
     __syncthreads();
 
     const u32x4 rs_a = make_rsrc(p.A, p.a_bytes);
-    const u32x4 rs_w = make_rsrc(p.W + (size_t)e * R * N * 2, (uint32_t)((size_t)R * N * 2));
+    const u32x4 rs_w = make_rsrc(p.W + (size_t)e * R * N * WES, (uint32_t)((size_t)R * N * WES));
 
     // ---------------- loader set-up: each wavefront issues 4 loads per operand per slab
     // K-major tile [256 rows][8 chunks]: load j covers rows 8j..8j+7; lane l lands on row 8j + l/8,
@@ -112,6 +117,14 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
                 int row = (wave * 4 + jj) * 8 + (lane >> 3);
                 int n = n0 + row;
                 qv[jj] = n < N ? (uint32_t)n * (uint32_t)R * 2 + ((lane & 7) ^ kmajor_key_relabelled(row)) * 16 : kVoffInvalid;
+            } else if constexpr (W_FP8) {
+                // bytes, [64 reduction rows][16 chunks]: load j (two per wavefront) covers rows 4j..4j+3; lane l lands
+                // on row 4j + l/16, physical chunk l%16; chunks are XORed with the low four bits of the row so that
+                // the 32 rows one transpose read touches spread over all banks
+                int row = (wave * 2 + (jj & 1)) * 4 + (lane >> 4);
+                int lchunk = (lane & 15) ^ (row & 15);
+                int n = n0 + lchunk * 16;
+                qv[jj] = (jj < 2 && n < N) ? (uint32_t)row * (uint32_t)N + n : kVoffInvalid;
             } else {
                 // [64 reduction rows][32 chunks]: load j covers rows 2j, 2j+1; lane l lands on row 2j + l/32,
                 // physical chunk l%32
@@ -126,11 +139,17 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
     auto issue = [&](int kt, int stage) {
         char *base = smem + stage * kDlStageBytes + wave * 4096;
         const uint32_t so_a = (uint32_t)kt * (BK * 2);
-        const uint32_t so_w = W_TRANS ? (uint32_t)kt * BK * (uint32_t)N * 2 : (uint32_t)kt * (BK * 2);
+        const uint32_t so_w = W_TRANS ? (uint32_t)kt * BK * (uint32_t)N * WES : (uint32_t)kt * (BK * 2);
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) direct_load16(rs_a, pv[jj], so_a, base + jj * 1024);
+        if constexpr (W_FP8) {
+            char *qbase = smem + stage * kDlStageBytes + kDlTileBytes + wave * 2048;
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) direct_load16(rs_w, qv[jj], so_w, base + kDlTileBytes + jj * 1024);
+            for (int jj = 0; jj < 2; ++jj) direct_load16(rs_w, qv[jj], so_w, qbase + jj * 1024);
+        } else {
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) direct_load16(rs_w, qv[jj], so_w, base + kDlTileBytes + jj * 1024);
+        }
     };
 
     // ---------------- fragment addresses
@@ -158,6 +177,9 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
             if constexpr (!W_TRANS) {
                 int row = wave_n0 + (a >> 2) * 16 + x * 4 + (a & 3);          // j = x (mod 2); + 8 rows per j/2
                 n_at[ks][x] = row * 128 + (((ks * 4 + g) ^ kmajor_key_relabelled(row)) << 4);
+            } else if constexpr (W_FP8) {
+                int row = ks * 32 + g * 8 + (a >> 1);                         // one read per fragment; x unused
+                n_at[ks][x] = row * 256 + (((wave_n0 >> 4) ^ (row & 15)) << 4) + (a & 1) * 8;
             } else {
                 int row = ks * 32 + g * 8 + x * 4 + (a >> 2);                 // x = h
                 n_at[ks][x] = row * 512 + (((wave_n0 >> 4) ^ tr_swizzle(row)) << 5) + (a & 3) * 8;
@@ -181,6 +203,9 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
             for (int j = 0; j < TN; ++j) {
                 if constexpr (!W_TRANS) {
                     nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][j & 1] + (j >> 1) * 1024);
+                } else if constexpr (W_FP8) {
+                    u32x2 q8 = lds_read_tr8(tile_n + (n_at[ks][0] ^ (j << 4)));      // chunk wave_n0/16 + j, j < 4
+                    nf[j] = fp8x8_to_bf16_chunk(q8[0], q8[1]);
                 } else {
                     // unit index wave_n0/16 + j: XOR with the swizzle commutes with adding j only bitwise,
                     // so fold j in by XOR on the unit field (wave_n0/16 is a multiple of 4, j < 4)

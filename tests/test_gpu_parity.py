@@ -375,3 +375,10 @@ def test_fp8_weight_gather_matches_dequantised_oracle():
     Y = hk.expert_gather_fp8w_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
     ref = O.gather_forward_fp8w(np64(case["X"]), Wq.view(torch.uint8).numpy(), scale.numpy(), case["Ind"].numpy())
     assert_close(Y, ref, torch.bfloat16, "fp8 weights odd")
+    # large product: 256 x 256 tiles, weight bytes staged in LDS as they are and widened after the transpose read
+    B, T, E, K, I, J = 3, 300, 5, 200, 192, 208
+    case = make_case(33, B, T, E, K, I, J, torch.bfloat16, replace=False)
+    Wq, scale = wl.quantize_fp8_weights(case["Wg"].float())
+    Y = hk.expert_gather_fp8w_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
+    ref = O.gather_forward_fp8w(np64(case["X"]), Wq.view(torch.uint8).numpy(), scale.numpy(), case["Ind"].numpy())
+    assert_close(Y, ref, torch.bfloat16, "fp8 weights large")
