@@ -1,6 +1,6 @@
 """Build recipe of the HIP library (``libegs_hip.so``) for gfx950.
 
-``python -m expertscattergather_amd.build`` compiles ``csrc/egs_lib.hip`` in-tree with hipcc.
+``python -m expertscattergather_amd.build`` compiles the ``csrc/*.hip`` translation units in-tree with hipcc.
 The library has no torch dependency; the Python side loads it with ctypes.
 """
 from __future__ import annotations
@@ -13,34 +13,45 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libegs_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["egs_lib.hip"]
-HEADERS = ["egs_device.h", "egs_rows_gemm.h", "egs_dw.h", "egs_scatter_aux.h"]
+SOURCES = ["egs_lib.hip", "egs_rows_launch.hip", "egs_dw_launch.hip"]
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-munsafe-fp-atomics",                      # fp32 atomic add as one hardware instruction
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed-fp32 VALU ops
     "-Wall", "-Wno-unused-function",
 ]
+NOISE = "is not a recognized feature for this target"
 
 
 def hipcc() -> str:
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 
-def build(verbose: bool = False, extra_flags=()) -> str:
-    """Compile the library (always recompiles) and return its path."""
-    cmd = [hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(os.path.dirname(HERE), "include"),
-           *[os.path.join(CSRC, s) for s in SOURCES], "-o", LIB_PATH]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    noise = "is not a recognized feature for this target"
-    out = "\n".join(l for l in res.stdout.splitlines() if noise not in l)
+    out = "\n".join(l for l in res.stdout.splitlines() if NOISE not in l)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
+
+
+def build(verbose: bool = False, extra_flags=()) -> str:
+    """Compile the library (always recompiles) and return its path.
+
+    The translation units are compiled side by side (object files under ``csrc/_obj``), then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+    obj_dir = os.path.join(CSRC, "_obj")
+    os.makedirs(obj_dir, exist_ok=True)
+    inc = ["-I", os.path.join(os.path.dirname(HERE), "include")]
+    objs = [os.path.join(obj_dir, s.replace(".hip", ".o")) for s in SOURCES]
+    cmds = [[hipcc(), *HIPCC_FLAGS, *extra_flags, *inc, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objs)]
+    with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
+        list(pool.map(lambda c: _run(c, verbose), cmds))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 

@@ -235,7 +235,7 @@ __global__ __launch_bounds__(kThreads) void dw_kernel(DwParams p)
 
 // dW(e,i,j) = sum_s part[s][e][i][j] in increasing s, rounded once to the output type and
 // written in the requested layout.
-__global__ __launch_bounds__(kThreads) void dw_reduce_kernel(const float *part, char *dW, int32_t S, int32_t E,
+static __global__ __launch_bounds__(kThreads) void dw_reduce_kernel(const float *part, char *dW, int32_t S, int32_t E,
                                                              int32_t I, int32_t J, int32_t out_dtype, int32_t dw_layout)
 {
     const size_t total = (size_t)E * I * J;

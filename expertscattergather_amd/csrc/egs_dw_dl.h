@@ -21,6 +21,8 @@
 
 namespace egs {
 
+constexpr int kDlThreads = 512;      // 8 wavefronts
+
 struct DwDlParams {
     DwParams d;               // i_tiles / j_tiles count 256-row and BQ-column tiles here
     uint32_t x_bytes, y_bytes;

@@ -1,53 +1,34 @@
-// Host side of the C ABI declared in include/egs_hip.h: argument validation, launch
-// planning (tile shapes, batch split of the weight gradient, workspace layout) and the
-// kernel launches.  No torch types, no device allocation, no synchronisation.
-#include <hip/hip_runtime.h>
-#include <stdint.h>
-#include <stdio.h>
-#include <string.h>
-
-#include "../../include/egs_hip.h"
+// Host side of the library: argument validation, workspace plans, kernel selection and the C ABI
+// declared in include/egs_hip.h.  The two template-heavy launch families (tiled rows products,
+// tiled weight gradients) live in egs_rows_launch.hip and egs_dw_launch.hip.
+#include "egs_host.h"
 #include "egs_device.h"
-#include "egs_rows_gemm.h"
-#include "egs_rows_gemm_dl.h"
-#include "egs_dw.h"
-#include "egs_dw_dl.h"
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
 
 using namespace egs;
+using namespace egs::host;
 
-namespace {
+namespace egs {
+namespace host {
 
-thread_local char g_hip_error[256] = "";
 bool g_force_generic = false;
-unsigned long long *g_dbg_times = nullptr;   // performance debugging: per-wavefront time stamps of the small rows kernel      // testing aid: skip the small-expert fast paths
+static thread_local char g_hip_error_buf[256] = "";
 
 int hip_fail(hipError_t err, const char *what)
 {
-    snprintf(g_hip_error, sizeof(g_hip_error), "%s: %s", what, hipGetErrorString(err));
+    snprintf(g_hip_error_buf, sizeof(g_hip_error_buf), "%s: %s", what, hipGetErrorString(err));
     return EGS_ERR_HIP;
 }
+const char *last_hip_error() { return g_hip_error_buf; }
 
-#define EGS_CHECK_LAUNCH(what)                                         \
-    do {                                                               \
-        hipError_t err__ = hipGetLastError();                          \
-        if (err__ != hipSuccess) return hip_fail(err__, what);         \
-    } while (0)
+}  // namespace host
+}  // namespace egs
 
-inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
-inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
-inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+namespace {
 
-int elem_size(int dtype)
-{
-    switch (dtype) {
-    case EGS_F32: return 4;
-    case EGS_F16: case EGS_BF16: return 2;
-    case EGS_FP8_E4M3: return 1;
-    default: return 0;
-    }
-}
+unsigned long long *g_dbg_times = nullptr;   // performance debugging: per-wavefront time stamps of the small rows kernel
+
 bool act_dtype_ok(int d) { return d == EGS_F32 || d == EGS_F16 || d == EGS_BF16; }
 bool ind_dtype_ok(int d) { return d >= EGS_IND_I16 && d <= EGS_IND_U8; }
 bool layout_ok(int l) { return l == EGS_W_EIJ || l == EGS_W_EJI; }
@@ -61,13 +42,6 @@ int check_dims(const egs_dims *d)
     if ((int64_t)d->B * d->K > INT32_MAX || (int64_t)d->E * d->K > INT32_MAX) return EGS_ERR_BAD_SHAPE;
     if ((int64_t)d->B * d->T > INT32_MAX) return EGS_ERR_BAD_SHAPE;
     return EGS_OK;
-}
-
-int grid_1d(size_t items, int cap = 8192)
-{
-    size_t g = (items + kThreads - 1) / kThreads;
-    if (g < 1) g = 1;
-    return (int)(g > (size_t)cap ? (size_t)cap : g);
 }
 
 // ------------------------------------------------------------------------------ plans
@@ -101,15 +75,6 @@ ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
     pl.bytes = at;
     return pl;
 }
-
-struct DwPlan {
-    int BI, BJ, BK, i_tiles, j_tiles, S, rows_per_split;   // general tiled kernel
-    bool small_ok;                                          // shape admits the small-expert kernel
-    int s_i_tiles, s_j_tiles, s_S, s_rows_per_split;        // its plan
-    bool big_ok;                                            // shape admits the direct-to-LDS kernel (256 x BQ tiles)
-    int b_bq, b_i_tiles, b_j_tiles, b_S, b_rows_per_split;  // its plan
-    size_t bytes;                                           // workspace covering whichever runs
-};
 
 DwPlan plan_dw(const egs_dims *d, int act_dtype)
 {
@@ -172,84 +137,6 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
         if (b2 > pl.bytes) pl.bytes = b2;
     }
     return pl;
-}
-
-// LDS the counting-sort routing table needs with `nw` wavefronts per batch element
-size_t csr_count_lds(int T, int nw) { return ((size_t)(nw + 1) * T + 1) * 4; }
-
-// ------------------------------------------------------------------------------ rows-GEMM dispatch
-template <class TT, int WES, bool GATHER, bool W_TRANS, int EPI>
-int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
-{
-    constexpr int BK = TT::ES == 4 ? 32 : 64;
-    const int Me = p.B * p.K;
-    if (Me == 0 || p.E == 0 || p.N == 0) return EGS_OK;
-    const int e_groups = ceil_div(p.E, 8);
-    // tile shape: 128 x 64 for narrow outputs, 256 x 256 (8 wavefronts) when the product is large
-    // enough to be bound by operand traffic (16-bit types), else 128 x 128
-    const bool big = TT::ES == 2 && EPI != EPI_ATOMIC_F32 && p.N >= 192 && Me >= 512 && p.R >= 128;
-    if (p.N <= 64) {
-        constexpr int BM = 128, BN = 64;
-        p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
-        int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
-        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-        hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 4, 1, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
-                           dim3(256), 0, s, p);
-    } else if (big) {
-        if constexpr (TT::ES == 2 && EPI != EPI_ATOMIC_F32) {
-            constexpr int BM = 256, BN = 256;
-            p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
-            int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
-            if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-            // well-formed shapes take the direct-to-LDS pipeline
-            const bool dl = !g_force_generic && p.R % kDlBK == 0 && p.N % (WES == 1 ? 16 : 8) == 0 && p.a_vec && p.w_vec &&
-                            p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && (WES == 1 || p.w_scale == nullptr) &&
-                            (WES == 2 || aligned_to(p.W, 16)) &&
-                            (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
-            if constexpr (WES == 2 || W_TRANS) {
-                if (dl) {
-                    p.csr_threads = kDlThreads;         // as many wavefronts as the histograms leave room for
-                    while (p.csr_threads > kWave && csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter)
-                        p.csr_threads >>= 1;
-                    if (GATHER || csr_count_lds(p.T, p.csr_threads / kWave) > (size_t)kDlSmemBytesScatter) p.csr_blocks = 0;
-                    grid += p.csr_blocks;
-                    p.csr_done = p.csr_blocks > 0;
-                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, p);
-                    EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
-                    return EGS_OK;
-                }
-            }
-            hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 4, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
-                               dim3(512), 0, s, p);
-        }
-    } else {
-        constexpr int BM = 128, BN = 128;
-        p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
-        int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
-        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-        hipLaunchKernelGGL((rows_gemm_kernel<TT, WES, BM, BN, BK, 2, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid),
-                           dim3(256), 0, s, p);
-    }
-    EGS_CHECK_LAUNCH("rows_gemm_kernel");
-    return EGS_OK;
-}
-
-template <class TT, bool GATHER, int EPI>
-int launch_rows_gemm_w(RowsGemmParams &p, bool w_trans, hipStream_t s)
-{
-    return w_trans ? launch_rows_gemm_cfg<TT, TT::ES, GATHER, true, EPI>(p, s)
-                   : launch_rows_gemm_cfg<TT, TT::ES, GATHER, false, EPI>(p, s);
-}
-
-template <bool GATHER, int EPI>
-int launch_rows_gemm(RowsGemmParams &p, int act_dtype, bool w_trans, hipStream_t s)
-{
-    switch (act_dtype) {
-    case EGS_F32: return launch_rows_gemm_w<ElemF32, GATHER, EPI>(p, w_trans, s);
-    case EGS_F16: return launch_rows_gemm_w<ElemF16, GATHER, EPI>(p, w_trans, s);
-    case EGS_BF16: return launch_rows_gemm_w<ElemBF16, GATHER, EPI>(p, w_trans, s);
-    default: return EGS_ERR_BAD_DTYPE;
-    }
 }
 
 // ------------------------------------------------------------------------------ small-expert fast paths
@@ -542,11 +429,7 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
             ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES : 0;
         p.a_bytes = span < (1ull << 31) ? (uint32_t)span : 0;
     }
-    if (w_dtype == EGS_FP8_E4M3) {
-        return w_trans ? launch_rows_gemm_cfg<ElemBF16, 1, true, true, EPI_STORE>(p, s)
-                       : launch_rows_gemm_cfg<ElemBF16, 1, true, false, EPI_STORE>(p, s);
-    }
-    return launch_rows_gemm<true, EPI_STORE>(p, act_dtype, w_trans, s);
+    return rows_gemm_gather(p, act_dtype, w_dtype == EGS_FP8_E4M3, w_trans, s);
 }
 
 // `dw` (optional): a weight gradient of the same call whose first pass may share the product
@@ -584,7 +467,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         EGS_CHECK_LAUNCH("fill_zero_f32_kernel");
         p.C = (char *)acc32;
         p.c_vec = 0;
-        return launch_rows_gemm<false, EPI_ATOMIC_F32>(p, act_dtype, w_trans, s);
+        return rows_gemm_scatter(p, act_dtype, w_trans, EPI_ATOMIC_F32, s);
     }
 
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
@@ -615,72 +498,11 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         // the routing table may ride along with the product launch (large shapes); otherwise it is a launch of its own
         p.csr_blocks = N > 0 ? d->B : 0; p.csr_done = 0;
         p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp; p.long_tab = long_tab;
-        rc = rows_f32 ? launch_rows_gemm<false, EPI_STORE_F32>(p, act_dtype, w_trans, s)
-                      : launch_rows_gemm<false, EPI_STORE>(p, act_dtype, w_trans, s);
+        rc = rows_gemm_scatter(p, act_dtype, w_trans, rows_f32 ? EPI_STORE_F32 : EPI_STORE, s);
         if (rc == EGS_OK && !p.csr_done) rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
     }
     if (rc != EGS_OK) return rc;
     return launch_segment_sum(rows, rows_f32, seg_off, perm, long_tab, long_part, Out, d, act_dtype, dw, s);
-}
-
-int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
-               int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout,
-               const DwPlan &pl, hipStream_t s)
-{
-    const size_t w_elems = (size_t)d->E * d->I * d->J;
-    const int ES = elem_size(act_dtype);
-    DwParams p;
-    memset(&p, 0, sizeof(p));
-    p.Xs = (const char *)Xs; p.Ys = (const char *)Ys; p.Ind = Ind;
-    p.part = (float *)workspace; p.dW = (char *)dW;
-    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.I = d->I; p.J = d->J;
-    p.ldx_b = ldx_b; p.ldx_t = ldx_t;
-    p.ind_dtype = ind_dtype;
-    p.x_vec = aligned_to(Xs, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
-    p.y_vec = aligned_to(Ys, 16) && ((int64_t)d->J * ES) % 16 == 0;
-    p.o_vec = aligned_to(dW, 16) && d->J % 4 == 0;
-    p.i_tiles = pl.i_tiles; p.j_tiles = pl.j_tiles; p.S = pl.S; p.rows_per_split = pl.rows_per_split;
-    p.out_dtype = out_dtype; p.dw_layout = dw_layout;
-    const uint64_t x_span = d->B > 0 && d->T > 0
-        ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES : 0;
-    const uint64_t y_span = (uint64_t)d->B * d->E * d->K * d->J * ES;
-    if (pl.big_ok && !g_force_generic && p.x_vec && p.y_vec && x_span < (1ull << 31) && y_span < (1ull << 31) &&
-        aligned_to(dW, 16)) {
-        DwDlParams q;
-        q.d = p;
-        q.d.i_tiles = pl.b_i_tiles; q.d.j_tiles = pl.b_j_tiles; q.d.S = pl.b_S; q.d.rows_per_split = pl.b_rows_per_split;
-        q.x_bytes = (uint32_t)x_span; q.y_bytes = (uint32_t)y_span;
-        const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.b_i_tiles * pl.b_j_tiles * pl.b_S;
-        if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-        if (act_dtype == EGS_F16) {
-            if (pl.b_bq == 256) hipLaunchKernelGGL((dw_dl_kernel<ElemF16, 256>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
-            else hipLaunchKernelGGL((dw_dl_kernel<ElemF16, 128>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
-        } else {
-            if (pl.b_bq == 256) hipLaunchKernelGGL((dw_dl_kernel<ElemBF16, 256>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
-            else hipLaunchKernelGGL((dw_dl_kernel<ElemBF16, 128>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
-        }
-        EGS_CHECK_LAUNCH("dw_dl_kernel");
-        if (pl.b_S > 1) {
-            hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s, (const float *)workspace,
-                               (char *)dW, pl.b_S, d->E, d->I, d->J, out_dtype, dw_layout);
-            EGS_CHECK_LAUNCH("dw_reduce_kernel");
-        }
-        return EGS_OK;
-    }
-    const int64_t grid = (int64_t)8 * ceil_div(d->E, 8) * pl.i_tiles * pl.j_tiles * pl.S;
-    if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-    switch (act_dtype) {
-    case EGS_F32: hipLaunchKernelGGL((dw_kernel<ElemF32, 128, 64, 32>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
-    case EGS_F16: hipLaunchKernelGGL((dw_kernel<ElemF16, 128, 64, 64>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
-    default: hipLaunchKernelGGL((dw_kernel<ElemBF16, 128, 64, 64>), dim3((unsigned)grid), dim3(kThreads), 0, s, p); break;
-    }
-    EGS_CHECK_LAUNCH("dw_kernel");
-    if (pl.S > 1) {
-        hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s, (const float *)workspace,
-                           (char *)dW, pl.S, d->E, d->I, d->J, out_dtype, dw_layout);
-        EGS_CHECK_LAUNCH("dw_reduce_kernel");
-    }
-    return EGS_OK;
 }
 
 int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,
@@ -792,7 +614,7 @@ const char *egs_status_string(int status)
     }
 }
 
-const char *egs_last_hip_error(void) { return g_hip_error; }
+const char *egs_last_hip_error(void) { return last_hip_error(); }
 
 void egs_set_force_generic(int on) { g_force_generic = on != 0; }
 void egs_set_debug_times(void *buf) { g_dbg_times = (unsigned long long *)buf; }

@@ -1,11 +1,14 @@
 // The rows x weight product of egs_rows_gemm.h for large, well-formed 16-bit shapes, built around
 // what gfx950 adds for this: 16-byte direct global->LDS loads and LDS transpose reads.
 //
-//   * 256 x 256 output tile, 64-deep slabs, 8 wavefronts (2 x 4), each 128 x 64 of the tile.
+//   * BM x 256 output tile (BM = 128 or 256), BK-deep slabs (32 or 64), BM/128 x 4 wavefronts, each
+//     128 x 64 of the tile.
 //   * Both operand slabs travel HBM/L2 -> LDS without touching registers (one buffer load per
-//     1 KB of a slab), two slabs in flight: the loads of slab k+1 are issued right after the
-//     barrier that publishes slab k and land while its 64 MFMAs per wavefront run.  One barrier
-//     per slab.
+//     1 KB of a slab), NSTAGE - 1 slabs in flight: the loads of slab k + NSTAGE - 1 are issued
+//     right after the barrier that publishes slab k and land while the MFMAs run.  One barrier
+//     per slab.  The shape in use is 256 x 256 x 64 with two stages (one 134 KB workgroup per CU, fewest
+//     bytes moved per flop); 128 x 256 x 32 with two or three stages (two or three workgroups per
+//     CU) compiles as well but measured slower on every benchmark configuration.
 //   * Rows that are fetched through Ind are just per-lane byte offsets into the buffer
 //     descriptor; rows that do not exist get an offset outside it and arrive as zeros.
 //   * K-major operands ([row][reduction]) are read back with 16-byte LDS reads (XOR swizzle set
@@ -26,36 +29,51 @@
 
 namespace egs {
 
-constexpr int kDlBM = 256, kDlBN = 256, kDlBK = 64, kDlThreads = 512;
-constexpr int kDlTileBytes = 256 * 64 * 2;              // one operand slab
-constexpr int kDlStageBytes = 2 * kDlTileBytes;
-constexpr int kDlSmemBytes = 2 * kDlStageBytes + kDlBM * 4 + kDlBM * 8;
-constexpr int kDlSmemBytesScatter = 150 * 1024;
+constexpr int kDlBN = 256;
+
+// LDS bytes of one workgroup: slab stages, then the row tables (4 + 8 bytes per tile row)
+__host__ __device__ constexpr int dl_stage_bytes(int BM, int BK) { return (BM + kDlBN) * BK * 2; }
+__host__ __device__ constexpr int dl_smem_bytes(int BM, int BK, int NSTAGE) { return NSTAGE * dl_stage_bytes(BM, BK) + BM * 12; }
+// the scatter variants of the one-workgroup-per-CU shape reserve more, so that the routing-table
+// workgroups riding along have room for eight wavefronts' histograms at T = 4096
+__host__ __device__ constexpr int dl_smem_bytes_scatter(int BM, int BK, int NSTAGE)
+{
+    return BM == 256 ? 150 * 1024 : dl_smem_bytes(BM, BK, NSTAGE);
+}
 
 // swizzle of the [reduction][column] tile: 32-byte units of a row are XORed with bits {0,1,3} of
 // the row number, which spreads the 16 rows one transpose read touches over all banks
 __device__ __forceinline__ int tr_swizzle(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
-// swizzle keys of the K-major tiles (XORed into the 16-byte chunk index of a 128-byte row).  The
-// row side reads 16 consecutive rows per 16 lanes; the weight side reads the relabelled rows
-// 16 c + 4 j + d (c, d = 0..3), whose distinguishing bits are 1, 4 and 5.
-__device__ __forceinline__ int kmajor_key_rows(int row) { return row & 7; }
-__device__ __forceinline__ int kmajor_key_relabelled(int row) { return (((row >> 4) & 3) << 1) | ((row >> 1) & 1); }
+// swizzle keys of the K-major tiles (XORed into the 16-byte chunk index of a row of CR chunks), chosen
+// so that the 16 lanes of one fragment read hit 16 different 16-byte bank groups.  The row side reads
+// 16 consecutive rows; the weight side reads the relabelled rows 16 c + 4 j + d (c, d = 0..3).
+template <int CR> __device__ __forceinline__ int kmajor_key_rows(int row) { return CR == 8 ? (row & 7) : ((row >> 2) & 3); }
+template <int CR> __device__ __forceinline__ int kmajor_key_relabelled(int row)
+{
+    return CR == 8 ? ((((row >> 4) & 3) << 1) | ((row >> 1) & 1)) : ((row >> 4) & 3);
+}
 
-template <class TT, int WES, bool GATHER, bool W_TRANS, int EPI>
-__global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams p)
+template <class TT, int WES, int BM, int BK, int NSTAGE, bool GATHER, bool W_TRANS, int EPI>
+__global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
 {
     static_assert(TT::ES == 2, "16-bit element types");
-    static_assert(WES == 2 || (WES == 1 && W_TRANS && TT::ID == 2), "fp8 weights: [reduction][column] layout, widened to bf16");
-    constexpr bool W_FP8 = (WES == 1);
     static_assert(EPI == EPI_STORE || EPI == EPI_STORE_F32, "plain stores only");
-    constexpr int BM = kDlBM, BN = kDlBN, BK = kDlBK;
+    static_assert(WES == 2 || (WES == 1 && W_TRANS && TT::ID == 2), "fp8 weights: [reduction][column] layout, widened to bf16");
+    static_assert((BM == 128 || BM == 256) && (BK == 32 || BK == 64) && (NSTAGE == 2 || NSTAGE == 3), "tile shapes");
+    constexpr bool W_FP8 = (WES == 1);
+    constexpr int BN = kDlBN;
+    constexpr int NT = BM * 2, NW = NT / 64;             // BM/128 x 4 wavefronts
     constexpr int TM = 8, TN = 4;                        // 16 x 16 tiles per wavefront: 128 x 64
+    constexpr int KSTEPS = BK / 32;
+    constexpr int CR = BK / 8;                           // 16-byte chunks per K-major row
+    constexpr int P_BYTES = BM * BK * 2, STAGE = dl_stage_bytes(BM, BK);
+    constexpr int PL = BM * CR / 64 / NW;                // loads per wavefront and slab: row side,
+    constexpr int QL = W_FP8 ? BK / 4 / NW : (W_TRANS ? BK / 2 / NW : BN * CR / 64 / NW);   // weight side
+    static_assert(PL >= 1 && QL >= 1 && PL + QL < 16, "loads per slab");
 
-    // two slab stages, then the row tables; the scatter variants reserve more so that the routing-table
-    // workgroups riding along have room for eight wavefronts' histograms at T = 4096
-    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? kDlSmemBytes : kDlSmemBytesScatter];
-    uint32_t *a_voff = reinterpret_cast<uint32_t *>(smem + 2 * kDlStageBytes);
-    int64_t *c_off = reinterpret_cast<int64_t *>(smem + 2 * kDlStageBytes + BM * 4);
+    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? dl_smem_bytes(BM, BK, NSTAGE) : dl_smem_bytes_scatter(BM, BK, NSTAGE)];
+    uint32_t *a_voff = reinterpret_cast<uint32_t *>(smem + NSTAGE * STAGE);
+    int64_t *c_off = reinterpret_cast<int64_t *>(smem + NSTAGE * STAGE + BM * 4);
 
     const int tid = (int)threadIdx.x;
     int block = (int)blockIdx.x;
@@ -103,53 +121,46 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
     const u32x4 rs_a = make_rsrc(p.A, p.a_bytes);
     const u32x4 rs_w = make_rsrc(p.W + (size_t)e * R * N * WES, (uint32_t)((size_t)R * N * WES));
 
-    // ---------------- loader set-up: each wavefront issues 4 loads per operand per slab
-    // K-major tile [256 rows][8 chunks]: load j covers rows 8j..8j+7; lane l lands on row 8j + l/8,
-    // physical chunk l%8, and therefore fetches logical chunk (l%8) ^ (l/8).
-    uint32_t pv[4], qv[4];
-    {
-        const int lc = (lane & 7) ^ (lane >> 3);
+    // ---------------- loader set-up.  One load covers 1 KB of a tile = 64 / CR rows of a K-major tile;
+    // lane l lands on row (64 / CR) j + l / CR, physical chunk l % CR, and therefore fetches the logical
+    // chunk (l % CR) ^ key(row).
+    uint32_t pv[PL], qv[QL];
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-            uint32_t ao = a_voff[(wave * 4 + jj) * 8 + (lane >> 3)];
-            pv[jj] = ao == kVoffInvalid ? kVoffInvalid : ao + lc * 16;
-            if constexpr (!W_TRANS) {
-                int row = (wave * 4 + jj) * 8 + (lane >> 3);
-                int n = n0 + row;
-                qv[jj] = n < N ? (uint32_t)n * (uint32_t)R * 2 + ((lane & 7) ^ kmajor_key_relabelled(row)) * 16 : kVoffInvalid;
-            } else if constexpr (W_FP8) {
-                // bytes, [64 reduction rows][16 chunks]: load j (two per wavefront) covers rows 4j..4j+3; lane l lands
-                // on row 4j + l/16, physical chunk l%16; chunks are XORed with the low four bits of the row so that
-                // the 32 rows one transpose read touches spread over all banks
-                int row = (wave * 2 + (jj & 1)) * 4 + (lane >> 4);
-                int lchunk = (lane & 15) ^ (row & 15);
-                int n = n0 + lchunk * 16;
-                qv[jj] = (jj < 2 && n < N) ? (uint32_t)row * (uint32_t)N + n : kVoffInvalid;
-            } else {
-                // [64 reduction rows][32 chunks]: load j covers rows 2j, 2j+1; lane l lands on row 2j + l/32,
-                // physical chunk l%32
-                int row = (wave * 4 + jj) * 2 + (lane >> 5);
-                int pc = lane & 31;
-                int lchunk = ((((pc >> 1) ^ tr_swizzle(row)) << 1) | (pc & 1));
-                int n = n0 + lchunk * 8;
-                qv[jj] = n < N ? ((uint32_t)row * (uint32_t)N + n) * 2 : kVoffInvalid;
-            }
+    for (int jj = 0; jj < PL; ++jj) {
+        const int row = (wave * PL + jj) * (64 / CR) + lane / CR;
+        const uint32_t ao = a_voff[row];
+        pv[jj] = ao == kVoffInvalid ? kVoffInvalid : ao + (((lane % CR) ^ kmajor_key_rows<CR>(row)) << 4);
+    }
+#pragma unroll
+    for (int jj = 0; jj < QL; ++jj) {
+        if constexpr (!W_TRANS) {
+            const int row = (wave * QL + jj) * (64 / CR) + lane / CR;
+            const int n = n0 + row;
+            qv[jj] = n < N ? (uint32_t)n * (uint32_t)R * 2 + (((lane % CR) ^ kmajor_key_relabelled<CR>(row)) << 4) : kVoffInvalid;
+        } else if constexpr (W_FP8) {
+            // bytes, [BK reduction rows][16 chunks]: a load covers 4 rows; lane l lands on row 4j + l/16, physical
+            // chunk l%16; chunks are XORed with the low four bits of the row so that the 32 rows one transpose
+            // read touches spread over all banks
+            const int row = (wave * QL + jj) * 4 + (lane >> 4);
+            const int n = n0 + ((lane & 15) ^ (row & 15)) * 16;
+            qv[jj] = n < N ? (uint32_t)row * (uint32_t)N + n : kVoffInvalid;
+        } else {
+            // [BK reduction rows][32 chunks]: a load covers 2 rows; lane l lands on row 2j + l/32, physical chunk l%32
+            const int row = (wave * QL + jj) * 2 + (lane >> 5);
+            const int pc = lane & 31;
+            const int n = n0 + ((((pc >> 1) ^ tr_swizzle(row)) << 1) | (pc & 1)) * 8;
+            qv[jj] = n < N ? ((uint32_t)row * (uint32_t)N + n) * 2 : kVoffInvalid;
         }
     }
     auto issue = [&](int kt, int stage) {
-        char *base = smem + stage * kDlStageBytes + wave * 4096;
+        char *pbase = smem + stage * STAGE + wave * (PL * 1024);
+        char *qbase = smem + stage * STAGE + P_BYTES + wave * (QL * 1024);
         const uint32_t so_a = (uint32_t)kt * (BK * 2);
         const uint32_t so_w = W_TRANS ? (uint32_t)kt * BK * (uint32_t)N * WES : (uint32_t)kt * (BK * 2);
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) direct_load16(rs_a, pv[jj], so_a, base + jj * 1024);
-        if constexpr (W_FP8) {
-            char *qbase = smem + stage * kDlStageBytes + kDlTileBytes + wave * 2048;
+        for (int jj = 0; jj < PL; ++jj) direct_load16(rs_a, pv[jj], so_a, pbase + jj * 1024);
 #pragma unroll
-            for (int jj = 0; jj < 2; ++jj) direct_load16(rs_w, qv[jj], so_w, qbase + jj * 1024);
-        } else {
-#pragma unroll
-            for (int jj = 0; jj < 4; ++jj) direct_load16(rs_w, qv[jj], so_w, base + kDlTileBytes + jj * 1024);
-        }
+        for (int jj = 0; jj < QL; ++jj) direct_load16(rs_w, qv[jj], so_w, qbase + jj * 1024);
     };
 
     // ---------------- fragment addresses
@@ -161,54 +172,64 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // row-side: row = wave_m0 + 16 i + a, physical chunk (4 ks + g) ^ (a & 7)
-    int m_at[2];
+    // row side: row = wave_m0 + 16 i + a (key does not depend on i), physical chunk (4 ks + g) ^ key
+    int m_at[KSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) m_at[ks] = (wave_m0 + a) * 128 + (((ks * 4 + g) ^ (a & 7)) << 4);
-    // weight-side, K-major: rows relabelled so that a lane ends up with 16 consecutive output columns
-    //   row(j) = wave_n0 + 16 (a/4) + 4 j + a%4
-    // weight-side, [reduction][column]: lane supplies row 32 ks + 8 g + 4 h + a/4 and columns
-    //   wave_n0 + 16 j + 4 (a%4) .. +3, so it receives column wave_n0 + 16 j + a
-    int n_at[2][2];
+    for (int ks = 0; ks < KSTEPS; ++ks)
+        m_at[ks] = (wave_m0 + a) * (BK * 2) + (((ks * 4 + g) ^ kmajor_key_rows<CR>(wave_m0 + a)) << 4);
+    // weight side, K-major: rows relabelled so that a lane ends up with 16 consecutive output columns,
+    //   row(j) = wave_n0 + 16 (a/4) + 4 j + a%4   (key does not depend on j)
+    // weight side, [reduction][column]: lane supplies row 32 ks + 8 g + 4 h + a/4 and columns
+    //   wave_n0 + 16 j + 4 (a%4) .. +3, so it receives column wave_n0 + 16 j + a   (fp8: row 32 ks + 8 g + a/2,
+    //   bytes 8 (a%2) .. +7 of the 16-byte chunk of tile j)
+    int n_at[KSTEPS][2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
+        for (int h = 0; h < 2; ++h) {
             if constexpr (!W_TRANS) {
-                int row = wave_n0 + (a >> 2) * 16 + x * 4 + (a & 3);          // j = x (mod 2); + 8 rows per j/2
-                n_at[ks][x] = row * 128 + (((ks * 4 + g) ^ kmajor_key_relabelled(row)) << 4);
+                const int row = wave_n0 + (a >> 2) * 16 + (a & 3);
+                n_at[ks][h] = row * (BK * 2) + (((ks * 4 + g) ^ kmajor_key_relabelled<CR>(row)) << 4);
             } else if constexpr (W_FP8) {
-                int row = ks * 32 + g * 8 + (a >> 1);                         // one read per fragment; x unused
-                n_at[ks][x] = row * 256 + (((wave_n0 >> 4) ^ (row & 15)) << 4) + (a & 1) * 8;
+                const int row = ks * 32 + g * 8 + (a >> 1);
+                n_at[ks][h] = row * 256 + (((wave_n0 >> 4) ^ (row & 15)) << 4) + (a & 1) * 8;
             } else {
-                int row = ks * 32 + g * 8 + x * 4 + (a >> 2);                 // x = h
-                n_at[ks][x] = row * 512 + (((wave_n0 >> 4) ^ tr_swizzle(row)) << 5) + (a & 3) * 8;
+                const int row = ks * 32 + g * 8 + h * 4 + (a >> 2);
+                n_at[ks][h] = row * 512 + (((wave_n0 >> 4) ^ tr_swizzle(row)) << 5) + (a & 3) * 8;
             }
         }
 
     const int nk = R / BK;
-    issue(0, 0);
-    for (int kt = 0; kt < nk; ++kt) {
-        wait_vmem<0>();
-        __syncthreads();            // slab kt visible to all; everyone is done reading the other stage
-        if (kt + 1 < nk) issue(kt + 1, (kt + 1) & 1);
-        const char *tile_m = smem + (kt & 1) * kDlStageBytes;
-        const char *tile_n = tile_m + kDlTileBytes;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+    for (int st = 0; st < NSTAGE - 1; ++st)
+        if (st < nk) issue(st, st);
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt) {
+        // slab kt has landed once at most the loads of the slabs issued after it are outstanding
+        if (NSTAGE == 3 && kt + 1 < nk) wait_vmem<(NSTAGE == 3 ? PL + QL : 0)>();
+        else wait_vmem<0>();
+        __syncthreads();            // slab kt visible to all; everyone is done reading the stage refilled next
+        if (kt + NSTAGE - 1 < nk) {
+            int fill = stage + NSTAGE - 1;
+            if (fill >= NSTAGE) fill -= NSTAGE;
+            issue(kt + NSTAGE - 1, fill);
+        }
+        const char *tile_m = smem + stage * STAGE;
+        const char *tile_n = tile_m + P_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
             u32x4 mf[TM], nf[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) mf[i] = *reinterpret_cast<const u32x4 *>(tile_m + m_at[ks] + i * 2048);
+            for (int i = 0; i < TM; ++i) mf[i] = *reinterpret_cast<const u32x4 *>(tile_m + m_at[ks] + i * (16 * BK * 2));
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (!W_TRANS) {
-                    nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][j & 1] + (j >> 1) * 1024);
+                    nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][0] + j * (4 * BK * 2));
                 } else if constexpr (W_FP8) {
                     u32x2 q8 = lds_read_tr8(tile_n + (n_at[ks][0] ^ (j << 4)));      // chunk wave_n0/16 + j, j < 4
                     nf[j] = fp8x8_to_bf16_chunk(q8[0], q8[1]);
                 } else {
-                    // unit index wave_n0/16 + j: XOR with the swizzle commutes with adding j only bitwise,
-                    // so fold j in by XOR on the unit field (wave_n0/16 is a multiple of 4, j < 4)
+                    // unit wave_n0/16 + j: wave_n0/16 is a multiple of 4 and j < 4, so j folds in by XOR
                     u32x2 lo = lds_read_tr16(tile_n + (n_at[ks][0] ^ (j << 5)));
                     u32x2 hi = lds_read_tr16(tile_n + (n_at[ks][1] ^ (j << 5)));
                     nf[j] = u32x4{lo[0], lo[1], hi[0], hi[1]};
@@ -219,6 +240,7 @@ __global__ __launch_bounds__(kDlThreads) void rows_gemm_dl_kernel(RowsGemmParams
 #pragma unroll
                 for (int j = 0; j < TN; ++j) mma_chunk<TT>(acc[i][j], nf[j], mf[i]);
         }
+        if (++stage == NSTAGE) stage = 0;
     }
 
     // ---------------- epilogue: 4 (transposed weights) or 16 (K-major weights) consecutive columns per lane and row

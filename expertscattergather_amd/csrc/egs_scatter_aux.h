@@ -80,7 +80,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, int lane)
 // General version: one wavefront per batch element does a counting sort.  Ranks inside a
 // 64-pick chunk come from ballots over the bits of the token id, not from atomics, so the
 // result does not depend on hardware ordering.  Works for any T and N; slow for large N.
-__global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
+static __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
                                                           int32_t *seg_off, int32_t *perm, int32_t *cnt_global,
                                                           int32_t *long_tab)
 {
@@ -268,7 +268,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
     emit_long_tokens(tok_start, T, N, long_tab, b, tid, nthreads);
 }
 
-__global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
+static __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
                                                          int32_t *seg_off, int32_t *perm, int32_t *rank_tmp,
                                                          int32_t *long_tab)
 {
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_
 // batch element sorts the keys (token << QB | q) with a bitonic network in LDS.  Keys are
 // unique, so the sorted order is the stable order by token.  NP = N rounded up to a power of
 // two; dynamic LDS = NP * 4 bytes.
-__global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
+static __global__ __launch_bounds__(1024) void csr_sort_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
                                                         int32_t NP, int32_t QB, int32_t *seg_off, int32_t *perm,
                                                         int32_t *long_tab)
 {
@@ -595,7 +595,7 @@ __global__ __launch_bounds__(kThreads) void segment_sum_kernel(SegSumParams sp)
 
 // zero n floats (the atomic mode's accumulator).  A kernel rather than a memset so that the
 // call sequence can be captured into a graph.  `vec` = dst is 16-byte aligned.
-__global__ __launch_bounds__(kThreads) void fill_zero_f32_kernel(float *dst, size_t n, int vec)
+static __global__ __launch_bounds__(kThreads) void fill_zero_f32_kernel(float *dst, size_t n, int vec)
 {
     const size_t n4 = vec ? n / 4 : 0;
     const size_t gid = (size_t)blockIdx.x * kThreads + threadIdx.x, stride = (size_t)gridDim.x * kThreads;
@@ -621,7 +621,7 @@ __global__ __launch_bounds__(kThreads) void downconvert_kernel(const float *src,
     for (size_t i = n4 * 4 + gid; i < n; i += stride) dst[i] = (uint16_t)f32_to_elem_bits<TT>(src[i]);
 }
 
-__global__ __launch_bounds__(kThreads) void validate_indices_kernel(const void *Ind, int32_t ind_dtype, int64_t n,
+static __global__ __launch_bounds__(kThreads) void validate_indices_kernel(const void *Ind, int32_t ind_dtype, int64_t n,
                                                                     int32_t T, int32_t *bad)
 {
     int local = 0;

@@ -423,7 +423,7 @@ __device__ __forceinline__ void dw_reduce4_body(const float *part, char *dW, int
 }
 
 
-__global__ __launch_bounds__(kThreads) void dw_reduce4_kernel(const float *part, char *dW, int32_t S, size_t total4,
+static __global__ __launch_bounds__(kThreads) void dw_reduce4_kernel(const float *part, char *dW, int32_t S, size_t total4,
                                                               int32_t out_dtype)
 {
     dw_reduce4_body(part, dW, S, total4, out_dtype, (int)blockIdx.x, (int)gridDim.x);
