@@ -24,6 +24,8 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
+# MI355X dense matrix peaks (TFLOP/s) of the arithmetic each configuration multiplies in
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
 
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
@@ -41,6 +43,7 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
+    ap.add_argument("--cold", action="store_true", help="also time each kernel with the caches flushed between launches")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch a 64 MiB device copy (3x) and the dominant kernel (5x), for rocprofv3 --pmc runs")
     return ap.parse_args()
@@ -79,8 +82,16 @@ def main():
         print(json.dumps({"pmc_probe": True, "copy_bytes_read": 64 << 20, "copy_bytes_written": 64 << 20}))
         return
 
+    fp8 = args.config == "C5"
+    if fp8:     # the configuration's weights: e4m3 bytes and a per-expert, per-column fp32 scale
+        Wq_c, scale_c = wl.quantize_fp8_weights(inp["Wg"].float())
+        Wq, Wscale = Wq_c.to(dev), scale_c.to(dev)
+
     def step():
-        Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        if fp8:
+            Y = hk.expert_gather_fp8w_forward(X, Wq, Wscale, Ind)
+        else:
+            Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
         out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
         if fwd_only:
             return Y, out
@@ -136,8 +147,9 @@ def main():
     mode = 0 if hk.get_scatter_mode() == "deterministic" else 1
     ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
-
     def k_gather():
+        if fp8:
+            return lib.egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), Wscale.data_ptr(), d, T * I, I, dt, 3, 2, 0, stream)
         return lib.egs_gather_gemm(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), None, d, T * I, I, dt, dt, 2, 0, stream)
 
     def k_scatter():
@@ -145,6 +157,9 @@ def main():
 
     def k_dw():
         return lib.egs_dw(X.data_ptr(), Y.data_ptr(), Ind.data_ptr(), dWbuf.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, dt, 2, 0, stream)
+
+    # a buffer larger than the 256 MB Infinity Cache, rewritten between launches for the cold numbers
+    flush = torch.empty(640 << 20, dtype=torch.uint8, device=dev) if args.cold else None
 
     def time_kernel(fn, reps):
         for _ in range(5):
@@ -158,28 +173,60 @@ def main():
         torch.cuda.synchronize()
         return start.elapsed_time(stop) * 1e-3 / reps
 
+    def time_kernel_cold(fn, reps):
+        total = 0.0
+        for _ in range(reps):
+            flush.add_(1)
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            fn()
+            stop.record()
+            torch.cuda.synchronize()
+            total += start.elapsed_time(stop) * 1e-3
+        return total / reps
+
     dims = cfg.dims
     gemm_bytes = wl.algorithmic_bytes(dims, act)
+    gather_bytes = wl.algorithmic_bytes(dims, act, w_bytes=1, fp8_scales=True) if fp8 else gemm_bytes
     dw_bytes = wl.algorithmic_bytes(dims, act, dw=True)
+    reps = args.kernel_reps if args.config in ("C1", "C2") else max(5, args.kernel_reps // 10)
     kernels = {
-        "gather_gemm": (time_kernel(k_gather, args.kernel_reps), gemm_bytes),
-        "gemm_scatter": (time_kernel(k_scatter, args.kernel_reps), gemm_bytes),
-        "dw": (time_kernel(k_dw, args.kernel_reps), dw_bytes),
+        "gather_gemm": (time_kernel(k_gather, reps), gather_bytes),
+        "gemm_scatter": (time_kernel(k_scatter, reps), gemm_bytes),
     }
+    if not fwd_only:
+        kernels["dw"] = (time_kernel(k_dw, reps), dw_bytes)
+    cold = None
+    if args.cold:
+        cold = {"gather_gemm": time_kernel_cold(k_gather, 10), "gemm_scatter": time_kernel_cold(k_scatter, 10)}
+        if not fwd_only:
+            cold["dw"] = time_kernel_cold(k_dw, 10)
     # gather_gemm is the kernel the whole path is named after and runs twice per step
     dom = "gather_gemm"
     dom_s, dom_bytes = kernels[dom]
     n_equiv = 2 if fwd_only else 6
-    chain_bytes = (2 if fwd_only else 4) * gemm_bytes + (0 if fwd_only else 2) * dw_bytes
-    chain_flops = n_equiv * wl.flops(dims)
+    chain_bytes = (gather_bytes + gemm_bytes) if fwd_only else 4 * gemm_bytes + 2 * dw_bytes
+    kflops = wl.flops(dims)
+    chain_flops = n_equiv * kflops
+    dtype_name = "bf16" if cfg.dtype == torch.bfloat16 else ("f16" if cfg.dtype == torch.float16 else "f32")
+    mfma_peak = MFMA_PEAK_TFLOPS[dtype_name]
+    # the roof that binds a kernel is the slower of "move the algorithmic bytes at 8 TB/s" and
+    # "do the flops at the dense matrix peak of the arithmetic type"
+    t_hbm, t_mfma = dom_bytes / (HBM_PEAK_GBPS * 1e9), kflops / (mfma_peak * 1e12)
+    bound = "hbm" if t_hbm >= t_mfma else "mfma"
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
     if not args.no_cpu_baseline:
         from oracle import torch_port as P
         cores = torch.get_num_threads()
-        Xc, Wgc, Wsc, dOc = (inp[k].float() for k in ("X", "Wg", "Ws", "dOut"))
-        Ic = inp["Ind"]
+        # bounded sample: the first nb batch elements (batch elements are independent), scaled to the full batch
+        nb = {"C1": B, "C2": B, "C3": 1, "C4": 4, "C5": 1}.get(args.config, B)
+        Xc, dOc = (inp[k][:nb].float() for k in ("X", "dOut"))
+        Wgc, Wsc = (inp[k].float() for k in ("Wg", "Ws"))
+        if fp8:
+            Wgc = Wq_c.float() * scale_c[:, None, :]        # dequantise-then-einsum, as the configuration's reference does
+        Ic = inp["Ind"][:nb]
 
         def cpu_step():
             if fwd_only:
@@ -195,8 +242,10 @@ def main():
             cpu_step()
             times.append(time.perf_counter() - t0)
         times.sort()
-        cpu = {"value": round(times[len(times) // 2] * 1e6, 1), "unit": "us", "cores": cores, "kind": "port",
-               "sample": f"median of {len(times)} full {cfg.name} steps of oracle/torch_port.py (torch CPU, fp32 arithmetic "
+        scale_to_full = B / nb
+        cpu = {"value": round(times[len(times) // 2] * 1e6 * scale_to_full, 1), "unit": "us", "cores": cores, "kind": "port",
+               "sample": f"median of {len(times)} {cfg.name} steps of oracle/torch_port.py over {nb} of {B} batch elements"
+                         f"{'' if nb == B else f' (time scaled by {scale_to_full:g})'} (torch CPU, fp32 arithmetic "
                          f"on the {str(cfg.dtype).split('.')[-1]}-rounded inputs)"}
 
     result = {
@@ -211,7 +260,7 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if cfg.dtype == torch.bfloat16 else str(cfg.dtype).split(".")[-1],
+        "dtype": dtype_name + (" (fp8 e4m3 weights)" if fp8 else ""),
         "data": "synthetic",
         "config": {"workload": f"{cfg.name}: B{B} T{T} E{E} K{K} I{I} J{J} {cfg.what}", "scatter_mode": hk.get_scatter_mode(),
                    "launch": "hip graph replay" if graph_s is not None else "eager"},
@@ -221,11 +270,20 @@ def main():
         "eager_us_per_step": round(eager_s * 1e6, 2),
         "graph_us_per_step": None if graph_s is None else round(graph_s * 1e6, 2),
         "kernel_us": {k: round(v[0] * 1e6, 2) for k, v in kernels.items()},
+        "kernel_us_cold": None if cold is None else {k: round(v * 1e6, 2) for k, v in cold.items()},
         "kernel_hbm_gbps": {k: round(v[1] / v[0] * 1e-9, 1) for k, v in kernels.items()},
-        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(dom_bytes / dom_s * 1e-9, 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
-                     "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_s * 1e6, 3)},
+        "kernel_hbm_frac": {k: round(v[1] / v[0] * 1e-9 / HBM_PEAK_GBPS, 4) for k, v in kernels.items()},
+        "kernel_tflops": {k: round(kflops / v[0] * 1e-12, 2) for k, v in kernels.items()},
+        "kernel_mfma_frac": {k: round(kflops / v[0] * 1e-12 / mfma_peak, 4) for k, v in kernels.items()},
+        "roofline": ({"bound": "hbm", "kernel": dom, "achieved": round(dom_bytes / dom_s * 1e-9, 1), "peak": HBM_PEAK_GBPS,
+                      "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4),
+                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                      "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_s * 1e6, 3)}
+                     if bound == "hbm" else
+                     {"bound": "mfma", "kernel": dom, "achieved": round(kflops / dom_s * 1e-12, 2), "peak": mfma_peak,
+                      "unit": "TFLOP/s", "frac": round(kflops / dom_s * 1e-12 / mfma_peak, 4),
+                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                      "algorithmic_flops": kflops, "avg_launch_us": round(dom_s * 1e6, 3)}),
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)

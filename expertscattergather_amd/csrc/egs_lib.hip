@@ -5,6 +5,7 @@
 #include "egs_device.h"
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
+#include "egs_scatter_fused.h"
 
 using namespace egs;
 using namespace egs::host;
@@ -401,6 +402,79 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
     return EGS_OK;
 }
 
+// ------------------------------------------------------------------------------ fused small-expert scatter
+template <class TT, bool W_NMAJOR, int KS>
+int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
+{
+    static size_t configured_plain = 64 * 1024, configured_dw = 64 * 1024;
+    if (dw != nullptr) {
+        const size_t need = lds > (size_t)kDwSmallLdsBytes ? lds : (size_t)kDwSmallLdsBytes;
+        if (need > configured_dw) {
+            hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_dw_kernel<TT, W_NMAJOR, KS>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
+            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_dw_kernel)");
+            configured_dw = need;
+        }
+        hipLaunchKernelGGL((scatter_fused_dw_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dw->blocks), dim3(kThreads), need, s, p,
+                           dw->q, blocks);
+        dw->done = true;
+    } else {
+        if (lds > configured_plain) {
+            hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_kernel<TT, W_NMAJOR, KS>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_kernel)");
+            configured_plain = lds;
+        }
+        hipLaunchKernelGGL((scatter_fused_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kThreads), lds, s, p);
+    }
+    EGS_CHECK_LAUNCH("scatter_fused_kernel");
+    return EGS_OK;
+}
+
+template <class TT, bool W_NMAJOR>
+int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
+{
+    switch (R) {
+    case 32: return launch_scatter_fused_one<TT, W_NMAJOR, 1>(p, lds, blocks, dw, s);
+    case 64: return launch_scatter_fused_one<TT, W_NMAJOR, 2>(p, lds, blocks, dw, s);
+    default: return launch_scatter_fused_one<TT, W_NMAJOR, 4>(p, lds, blocks, dw, s);
+    }
+}
+
+// GEMM-scatter of small experts in one kernel (product rows stay in LDS); `used` reports whether the
+// shape qualified.  Both scatter modes take it: it is bitwise reproducible and needs no workspace.
+int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
+                  int w_layout, SmallDwJob *dw, hipStream_t s, bool &used)
+{
+    used = false;
+    const int R = d->J, N = d->I;
+    const int64_t NP = (int64_t)d->E * d->K;
+    if (g_force_generic || act_dtype == EGS_F32 || !(R == 32 || R == 64 || R == 128)) return EGS_OK;
+    if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 1024 || d->T < 1 || d->B < 1) return EGS_OK;
+    const size_t lds = scatter_fused_lds(d->T, (int)NP);
+    if (lds > 156 * 1024) return EGS_OK;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 8)) return EGS_OK;
+    if ((uint64_t)d->B * NP * R * 2 > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32) return EGS_OK;
+    const int slices = N / kFusedCols;
+    const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
+    if (blocks > INT32_MAX / 2 || (int64_t)d->B * slices < 8) return EGS_OK;        // too few workgroups to be worth it
+    ScatterFusedParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)Y; p.W = (const char *)W; p.Ind = Ind; p.out = (char *)Out;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
+    p.ind_dtype = ind_dtype;
+    p.slices = slices;
+    p.perm_at = (int32_t)(NP * kFusedCols * 4);
+    p.cnt_at = p.perm_at + (int32_t)(NP * 4);
+    used = true;
+    const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
+    if (act_dtype == EGS_F16)
+        return nmajor ? launch_scatter_fused_ks<ElemF16, true>(p, R, lds, (int)blocks, dw, s)
+                      : launch_scatter_fused_ks<ElemF16, false>(p, R, lds, (int)blocks, dw, s);
+    return nmajor ? launch_scatter_fused_ks<ElemBF16, true>(p, R, lds, (int)blocks, dw, s)
+                  : launch_scatter_fused_ks<ElemBF16, false>(p, R, lds, (int)blocks, dw, s);
+}
+
 // ------------------------------------------------------------------------------ implementations
 int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
                      const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
@@ -468,6 +542,12 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         p.C = (char *)acc32;
         p.c_vec = 0;
         return rows_gemm_scatter(p, act_dtype, w_trans, EPI_ATOMIC_F32, s);
+    }
+
+    {   // small experts: everything in one kernel
+        bool used = false;
+        const int rc_fused = scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, s, used);
+        if (used) return rc_fused;
     }
 
     // routing table (picks in token order) + product rows in pick order, then one fixed-order

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
         // builds it here (csr_threads of the workgroup, histograms in the slab buffers) instead of in a launch of its own
         if (block < p.csr_blocks) {
             if (tid >= p.csr_threads) return;
-            csr_count_body(reinterpret_cast<int32_t *>(smem), block, tid, p.csr_threads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
+            csr_count_body(reinterpret_cast<int32_t *>(smem), block, block, tid, p.csr_threads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
                            p.seg_off, p.perm, p.rank_tmp, p.long_tab);
             return;
         }

@@ -140,8 +140,11 @@ static __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind
 // histogram (ballot matching inside each 64-pick chunk, no atomics), then the per-token counts
 // are prefix-summed over wavefronts and over tokens, and every pick goes to
 //   start of its token + picks of that token in earlier slices + rank inside its slice.
-// LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch.
-__device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, int nthreads, const void *Ind,
+// LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch (only touched when a wavefront's
+// slice exceeds 512 picks).  Picks are read at batch element `b`; results are written at batch element
+// `out_b` of seg_off / perm (a caller that keeps them in LDS passes 0 and seg_off = nullptr: the
+// offsets are left in sh_cnt[NW * T ..]).
+__device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b, int tid, int nthreads, const void *Ind,
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
                                                int32_t *perm, int32_t *rank_tmp, int32_t *long_tab)
 {
@@ -149,7 +152,8 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
     const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
     int32_t *hist = sh_cnt + (size_t)wave * T;          // this wavefront's counters
     int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
-    const int64_t base_pick = (int64_t)b * N;
+    const int64_t base_pick = (int64_t)b * N;           // where this batch element's picks start in Ind
+    const int64_t out_pick = (int64_t)out_b * N;        // ... and in perm / rank_tmp
     const int slice = ((N + NW - 1) / NW + 63) & ~63;
     const int q_begin = wave * slice, q_end = min(N, q_begin + slice);
     const bool in_regs = slice <= MAXC * kWave;
@@ -203,7 +207,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
             for (int c = 0; c < MAXC; ++c) {
                 if (q0 + c * kWave >= q_end) break;
                 const int r = rank_chunk(tk[c]);
-                if (tk[c] >= 0) rank_tmp[base_pick + q0 + c * kWave + lane] = r;
+                if (tk[c] >= 0) rank_tmp[out_pick + q0 + c * kWave + lane] = r;
             }
         }
     }
@@ -245,11 +249,12 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
         if (tid == 0) tok_start[T] = total;
     }
     __syncthreads();
-    for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)b * (T + 1) + t] = tok_start[t];
+    if (seg_off != nullptr)
+        for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)out_b * (T + 1) + t] = tok_start[t];
     if (in_regs) {
 #pragma unroll
         for (int c = 0; c < MAXC; ++c)
-            if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rk[c]] = q_begin + c * kWave + lane;
+            if (tk[c] >= 0) perm[out_pick + tok_start[tk[c]] + hist[tk[c]] + rk[c]] = q_begin + c * kWave + lane;
     } else {
         for (int q0 = q_begin; q0 < q_end; q0 += MAXC * kWave) {
             int32_t rr[MAXC];
@@ -257,15 +262,15 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int tid, 
             for (int c = 0; c < MAXC; ++c) {
                 const int q = q0 + c * kWave + lane;
                 const int32_t t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);
-                rr[c] = rank_tmp[base_pick + min(q, N - 1)];
+                rr[c] = rank_tmp[out_pick + min(q, N - 1)];
                 tk[c] = q < q_end ? t : -1;
             }
 #pragma unroll
             for (int c = 0; c < MAXC; ++c)
-                if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + hist[tk[c]] + rr[c]] = q0 + c * kWave + lane;
+                if (tk[c] >= 0) perm[out_pick + tok_start[tk[c]] + hist[tk[c]] + rr[c]] = q0 + c * kWave + lane;
         }
     }
-    emit_long_tokens(tok_start, T, N, long_tab, b, tid, nthreads);
+    emit_long_tokens(tok_start, T, N, long_tab, out_b, tid, nthreads);
 }
 
 static __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
@@ -273,7 +278,7 @@ static __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind,
                                                          int32_t *long_tab)
 {
     extern __shared__ int32_t sh_cnt_dyn[];
-    csr_count_body(sh_cnt_dyn, (int)blockIdx.x, (int)threadIdx.x, (int)blockDim.x, Ind, ind_dtype, T, N, seg_off, perm,
+    csr_count_body(sh_cnt_dyn, (int)blockIdx.x, (int)blockIdx.x, (int)threadIdx.x, (int)blockDim.x, Ind, ind_dtype, T, N, seg_off, perm,
                    rank_tmp, long_tab);
 }
 

@@ -55,7 +55,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     static_assert(!(GATHER && OUT_F32), "gather results are stored in the element type");
     if constexpr (!GATHER) {
         if (block < p.csr_blocks) {
-            csr_count_body(sh_cnt_small, block, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
+            csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
                            p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
             return;
         }
@@ -250,13 +250,14 @@ struct SmallDwParams {
 };
 
 constexpr int kDwSmallMaxRows = 1024;   // picks of one workgroup (row offsets staged in LDS)
+constexpr int kDwSmallLdsBytes = 4 * 64 * 64 * 4;
 
 // Requirements: 2-byte elements, I % 8 == 0, J % 8 == 0, rows 16-byte aligned, spans < 4 GiB,
 // rows_per_split <= kDwSmallMaxRows.
 template <class TT>
-__device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int block)
+__device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int block, float *red)
 {
-    __shared__ __attribute__((aligned(16))) float red[4 * 64 * 64];       // 64 KB: one tile per wavefront
+    // red: kDwSmallLdsBytes of 16-byte aligned LDS, one 64 x 64 tile per wavefront
     uint32_t *xoff_lds = reinterpret_cast<uint32_t *>(red);              // reused before the reduction:
     uint32_t *yoff_lds = xoff_lds + kDwSmallMaxRows;                      //   row byte offsets, 0xFFFFFFFF = no row
 
@@ -397,7 +398,8 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
 template <class TT>
 __global__ __launch_bounds__(kThreads) void dw_small_kernel(SmallDwParams p)
 {
-    dw_small_body<TT>(p, (int)blockIdx.x);
+    __shared__ __attribute__((aligned(16))) float red[kDwSmallLdsBytes / 4];
+    dw_small_body<TT>(p, (int)blockIdx.x, red);
 }
 
 // dW = sum_s part[s] in increasing s, rounded once; partials already have the output's layout.
@@ -437,8 +439,9 @@ template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
 __global__ __launch_bounds__(kThreads) void rows_dw_small_kernel(SmallRowsParams p, SmallDwParams q, int rows_blocks)
 {
     extern __shared__ int32_t sh_dyn_fused[];
+    __shared__ __attribute__((aligned(16))) float red[kDwSmallLdsBytes / 4];
     if ((int)blockIdx.x < rows_blocks) rows_small_body<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>(p, (int)blockIdx.x, sh_dyn_fused);
-    else dw_small_body<TT>(q, (int)blockIdx.x - rows_blocks);
+    else dw_small_body<TT>(q, (int)blockIdx.x - rows_blocks, red);
 }
 
 // segment sums of a scatter and the second pass of a weight gradient in one launch:

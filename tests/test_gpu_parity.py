@@ -73,6 +73,8 @@ SMALL_SHAPES = [
     (9, 40, 12, 33, 128, 32),     # K = 33
     (2, 700, 8, 20, 32, 64),      # long T: accumulators of one expert group fill the LDS
     (3, 64, 16, 16, 64, 56),      # J not a multiple of 16 (gather columns), scatter takes the general path
+    (8, 60, 6, 20, 64, 128),      # reduction 128 on the one-kernel scatter, ragged 16-pick tiles
+    (4, 300, 40, 25, 96, 32),     # 1000 picks per batch element, three 32-column slices
 ]
 
 
