@@ -328,6 +328,19 @@ __device__ __forceinline__ void transpose4x4_32b(const u32x4 (&in)[4], u32x4 (&o
         for (int r = 0; r < 4; ++r) out[c][r] = in[r][c];
 }
 
+// Lane transposition 16 x 4 -> 4 x 16: lane 16 g + a receives what lane 4 a + g holds.  A global load in
+// which lanes 4a .. 4a+3 fetch four consecutive 16-byte chunks of row a is what the memory pipeline
+// coalesces (one 64-byte access per row instead of four 16-byte ones); an MFMA operand wants row a's
+// chunk g in lane 16 g + a.  Four cross-lane moves (no LDS storage involved) convert one into the other.
+__device__ __forceinline__ u32x4 lanes_4a_g_to_16g_a(const u32x4 &v, int lane)
+{
+    const int src = ((lane & 15) << 2 | (lane >> 4)) << 2;       // byte address of the source lane
+    u32x4 r;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) r[x] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)v[x]);
+    return r;
+}
+
 // workgroup id -> (expert, tile): consecutive workgroup ids land on consecutive XCDs (8 per
 // device), so expert = 8*group + (id % 8) keeps all tiles of one expert on one XCD and its
 // weight tile in that XCD's L2.

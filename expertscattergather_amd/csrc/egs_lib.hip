@@ -415,7 +415,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
             if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_dw_kernel)");
             configured_dw = need;
         }
-        hipLaunchKernelGGL((scatter_fused_dw_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dw->blocks), dim3(kThreads), need, s, p,
+        hipLaunchKernelGGL((scatter_fused_dw_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dw->blocks), dim3(kFusedThreads), need, s, p,
                            dw->q, blocks);
         dw->done = true;
     } else {
@@ -425,7 +425,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
             if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_kernel)");
             configured_plain = lds;
         }
-        hipLaunchKernelGGL((scatter_fused_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kThreads), lds, s, p);
+        hipLaunchKernelGGL((scatter_fused_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     }
     EGS_CHECK_LAUNCH("scatter_fused_kernel");
     return EGS_OK;

@@ -143,10 +143,15 @@ static __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind
 // LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch (only touched when a wavefront's
 // slice exceeds 512 picks).  Picks are read at batch element `b`; results are written at batch element
 // `out_b` of seg_off / perm (a caller that keeps them in LDS passes 0 and seg_off = nullptr: the
-// offsets are left in sh_cnt[NW * T ..]).
+// offsets are left in sh_cnt[NW * T ..]).  `after_token_loads` runs right after the token loads have been
+// issued (a caller's own prefetches belong there: the tokens are the sort's critical path).
+struct NoPrefetch { __device__ __forceinline__ void operator()() const {} };
+
+template <class AfterTokenLoads = NoPrefetch>
 __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b, int tid, int nthreads, const void *Ind,
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
-                                               int32_t *perm, int32_t *rank_tmp, int32_t *long_tab)
+                                               int32_t *perm, int32_t *rank_tmp, int32_t *long_tab,
+                                               AfterTokenLoads after_token_loads = AfterTokenLoads())
 {
     constexpr int MAXC = 8;                             // 64-pick chunks whose tokens (and ranks) are held in registers at a time
     const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
@@ -167,6 +172,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
         tk[c] = (in_regs && q < q_end) ? t : -1;
         rk[c] = 0;
     }
+    after_token_loads();        // whatever else the caller wants in flight while the tokens travel
 
     for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
     __syncthreads();

@@ -7,7 +7,7 @@
 //   (0) sorts the picks of b by token in LDS (the counting sort of csr_count_body; the slices of
 //       one batch element repeat it, which is cheaper than a launch of its own),
 //   (1) multiplies every pick's row by its expert's weight slice on the MFMAs (operands straight
-//       from global memory into registers, several (expert, 16-pick) units in flight per wavefront)
+//       from global memory into registers, several (expert, 32-pick) units in flight per wavefront)
 //       and parks the fp32 products in LDS, one 128-byte row per pick,
 //   (2) walks each token's segment of the table, adds its product rows in table order in fp32,
 //       rounds once and writes the output row slice (tokens nobody picked become zero).
@@ -28,6 +28,7 @@
 namespace egs {
 
 constexpr int kFusedCols = 32;          // output columns per workgroup
+constexpr int kFusedThreads = 512;      // 8 wavefronts: enough units in flight to cover the memory latency in two rounds
 
 struct ScatterFusedParams {
     const char *A;          // [B,E,K,R] dense rows, 16-bit
@@ -40,10 +41,10 @@ struct ScatterFusedParams {
     int32_t perm_at, cnt_at;    // byte offsets of the table and of the sort's counters in dynamic LDS (rows start at 0)
 };
 
-// LDS bytes: product rows, table, counters of the sort (4 wavefronts)
+// LDS bytes: product rows, table, counters of the sort (one histogram per wavefront + offsets)
 __host__ __device__ inline size_t scatter_fused_lds(int T, int NP)
 {
-    return (size_t)NP * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)5 * T + 1) * 4 + 64;
+    return (size_t)NP * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)(kFusedThreads / 64 + 1) * T + 1) * 4 + 64;
 }
 
 template <class TT, bool W_NMAJOR, int KS>
@@ -51,7 +52,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 {
     static_assert(TT::ES == 2, "16-bit element types");
     constexpr int R = 32 * KS;
-    constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 16-pick) units in flight per wavefront
+    constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 32-pick) units in flight per wavefront
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int a = lane & 15, g = lane >> 4;
     // slices of one batch element sit on one XCD (ids congruent modulo 8 share an XCD), so that its
@@ -65,28 +66,34 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     float *rows = reinterpret_cast<float *>(smem);
     int32_t *perm = reinterpret_cast<int32_t *>(smem + p.perm_at);
     int32_t *cnt = reinterpret_cast<int32_t *>(smem + p.cnt_at);
-    const int32_t *seg = cnt + 4 * T;                   // token offsets left there by the sort
+    constexpr int NWV = kFusedThreads / 64;
+    const int32_t *seg = cnt + NWV * T;                 // token offsets left there by the sort
 
-    // ---------------- (1) units of work of this wavefront: (expert, 16-pick row tile)
-    const int KT = (K + 15) >> 4;
-    const int units = E * KT;
-    struct Unit { u32x4 y[KS]; u32x4 w[W_NMAJOR ? 2 * KS : 2 * KS]; };
+    // ---------------- (1) units of work of this wavefront: (expert, pair of 16-pick row tiles); the weight
+    // fragments of a unit serve both row tiles
+    const int KT2 = (K + 31) >> 5;
+    const int units = E * KT2;
+    struct Unit { u32x4 y[2][KS]; u32x4 w[2 * KS]; };
     Unit buf[kFusedDepth];
     const uint32_t a_base_b = (uint32_t)b * (uint32_t)NP * R * 2;
     auto load_unit = [&](Unit &u, int unit) {
         unit = min(unit, units - 1);                    // unconditional loads; surplus units are not stored
-        const int e = unit / KT, rt = unit - e * KT;
-        const int k = min(rt * 16 + a, K - 1);
-        const char *yrow = p.A + a_base_b + (uint32_t)((e * K + k) * R * 2);
+        const int e = unit / KT2, rp = unit - e * KT2;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) u.y[ks] = *reinterpret_cast<const u32x4 *>(yrow + (ks * 32 + g * 8) * 2);
+        for (int h = 0; h < 2; ++h) {
+            // coalesced: lanes 4r .. 4r+3 fetch four consecutive chunks of row r; transposed to operand order at use
+            const int k = min(rp * 32 + h * 16 + (lane >> 2), K - 1);
+            const char *yrow = p.A + a_base_b + (uint32_t)((e * K + k) * R * 2);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) u.y[h][ks] = *reinterpret_cast<const u32x4 *>(yrow + (ks * 32 + (lane & 3) * 8) * 2);
+        }
         if constexpr (!W_NMAJOR) {
             // [E,N,R]: the lane's output column is a row of W
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
-                const char *wrow = p.W + ((size_t)e * N + c0 + ct * 16 + a) * (R * 2);
+                const char *wrow = p.W + ((size_t)e * N + c0 + ct * 16 + (lane >> 2)) * (R * 2);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) u.w[ct * KS + ks] = *reinterpret_cast<const u32x4 *>(wrow + (ks * 32 + g * 8) * 2);
+                for (int ks = 0; ks < KS; ++ks) u.w[ct * KS + ks] = *reinterpret_cast<const u32x4 *>(wrow + (ks * 32 + (lane & 3) * 8) * 2);
             }
         } else {
             // [E,R,N]: 8 (reduction) x 2 (columns 2a, 2a+1) blocks, transposed in registers below; raw rows kept here
@@ -101,13 +108,15 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     };
     auto compute_unit = [&](const Unit &u, int unit) {
         if (unit >= units) return;
-        const int e = unit / KT, rt = unit - e * KT;
-        f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+        const int e = unit / KT2, rp = unit - e * KT2;
+        f32x4 acc[2][2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) { acc[h][0] = f32x4{0.f, 0.f, 0.f, 0.f}; acc[h][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             u32x4 wf[2];
             if constexpr (!W_NMAJOR) {
-                wf[0] = u.w[ks]; wf[1] = u.w[KS + ks];
+                wf[0] = lanes_4a_g_to_16g_a(u.w[ks], lane); wf[1] = lanes_4a_g_to_16g_a(u.w[KS + ks], lane);
             } else {
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
@@ -116,45 +125,52 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
                     wf[1][pp] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);     // column 2a+1
                 }
             }
-            mma_chunk<TT>(acc[0], wf[0], u.y[ks]);
-            mma_chunk<TT>(acc[1], wf[1], u.y[ks]);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const u32x4 yf = lanes_4a_g_to_16g_a(u.y[h][ks], lane);
+                mma_chunk<TT>(acc[h][0], wf[0], yf);
+                mma_chunk<TT>(acc[h][1], wf[1], yf);
+            }
         }
-        // lane (a, g) holds, for pick k = 16 rt + a, slice columns
+        // lane (a, g) holds, for pick k = 32 rp + 16 h + a, slice columns
         //   [E,N,R]: 16 ct + 4 g + r            -> chunk 4 ct + g of the row
         //   [E,R,N]: 2 (4 g + r) + ct = 8 g + 2 r + ct -> chunks 2 g, 2 g + 1 after interleaving the two tiles
-        const int k = rt * 16 + a;
-        if (k < K) {
-            const int q = e * K + k;
-            f32x4 *row = reinterpret_cast<f32x4 *>(rows + (size_t)q * kFusedCols);
-            if constexpr (!W_NMAJOR) {
-                row[(g) ^ (q & 7)] = acc[0];
-                row[(4 + g) ^ (q & 7)] = acc[1];
-            } else {
-                row[(2 * g) ^ (q & 7)] = f32x4{acc[0][0], acc[1][0], acc[0][1], acc[1][1]};
-                row[(2 * g + 1) ^ (q & 7)] = f32x4{acc[0][2], acc[1][2], acc[0][3], acc[1][3]};
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = rp * 32 + h * 16 + a;
+            if (k < K) {
+                const int q = e * K + k;
+                f32x4 *row = reinterpret_cast<f32x4 *>(rows + (size_t)q * kFusedCols);
+                if constexpr (!W_NMAJOR) {
+                    row[(g) ^ (q & 7)] = acc[h][0];
+                    row[(4 + g) ^ (q & 7)] = acc[h][1];
+                } else {
+                    row[(2 * g) ^ (q & 7)] = f32x4{acc[h][0][0], acc[h][1][0], acc[h][0][1], acc[h][1][1]};
+                    row[(2 * g + 1) ^ (q & 7)] = f32x4{acc[h][0][2], acc[h][1][2], acc[h][0][3], acc[h][1][3]};
+                }
             }
         }
     };
 
-    // first units go in flight, then the sort runs while they travel
+    // ---------------- (0) routing table of batch element b in LDS; the first units' operands go in flight
+    // right behind the sort's token loads and travel while it runs
+    csr_count_body(cnt, b, 0, tid, kFusedThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr, [&]() {
 #pragma unroll
-    for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + 4 * d);
+        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d);
+    });
 
-    // ---------------- (0) routing table of batch element b in LDS
-    csr_count_body(cnt, b, 0, tid, kThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr);
-
-    for (int u0 = wave; u0 < units; u0 += 4 * kFusedDepth) {
+    for (int u0 = wave; u0 < units; u0 += NWV * kFusedDepth) {
 #pragma unroll
         for (int d = 0; d < kFusedDepth; ++d) {
-            compute_unit(buf[d], u0 + 4 * d);
-            load_unit(buf[d], u0 + 4 * d + 4 * kFusedDepth);
+            compute_unit(buf[d], u0 + NWV * d);
+            load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth);
         }
     }
     __syncthreads();
 
     // ---------------- (2) per token: add its product rows in table order; 8 threads x 4 columns per token
     const int cc = tid & 7;
-    for (int t = tid >> 3; t < T; t += kThreads >> 3) {
+    for (int t = tid >> 3; t < T; t += kFusedThreads >> 3) {
         const int s0 = seg[t], s1 = seg[t + 1];
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int s = s0; s < s1; s += 4) {
@@ -176,7 +192,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 }
 
 template <class TT, bool W_NMAJOR, int KS>
-__global__ __launch_bounds__(kThreads) void scatter_fused_kernel(ScatterFusedParams p)
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_kernel(ScatterFusedParams p)
 {
     extern __shared__ __attribute__((aligned(16))) char smem_fused[];
     scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused);
@@ -185,11 +201,15 @@ __global__ __launch_bounds__(kThreads) void scatter_fused_kernel(ScatterFusedPar
 // the same with the first pass of a small weight gradient of the same backward call in the launch:
 // workgroups [0, fused_blocks) run the scatter, the rest the weight gradient
 template <class TT, bool W_NMAJOR, int KS>
-__global__ __launch_bounds__(kThreads) void scatter_fused_dw_kernel(ScatterFusedParams p, SmallDwParams q, int fused_blocks)
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_dw_kernel(ScatterFusedParams p, SmallDwParams q, int fused_blocks)
 {
     extern __shared__ __attribute__((aligned(16))) char smem_fused_dw[];
-    if ((int)blockIdx.x < fused_blocks) scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused_dw);
-    else dw_small_body<TT>(q, (int)blockIdx.x - fused_blocks, reinterpret_cast<float *>(smem_fused_dw));
+    if ((int)blockIdx.x < fused_blocks) {
+        scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused_dw);
+    } else {
+        if ((int)threadIdx.x >= kThreads) return;       // the weight gradient is written for four wavefronts
+        dw_small_body<TT>(q, (int)blockIdx.x - fused_blocks, reinterpret_cast<float *>(smem_fused_dw));
+    }
 }
 
 }  // namespace egs
