@@ -145,14 +145,20 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
         }
     }
 
-    // row fragments: lane (a, g) of row tile tq supplies elements [32*ks + 8*g, +8) of row 16*tq + a
+    // row fragments: lane (a, g) of row tile tq supplies elements [32*ks + 8*g, +8) of row 16*tq + a.  They are
+    // fetched coalesced (lanes 4r .. 4r+3 take four consecutive 16-byte chunks of row 16*tq + r: one 64-byte
+    // access per row instead of four scattered 16-byte ones) and moved to operand order across lanes.
     u32x4 xf[TQ][KS];
 #pragma unroll
     for (int tq = 0; tq < TQ; ++tq) {
-        const uint32_t xo = (uint32_t)__shfl((int)aoff, tq * 16 + a, kWave) + (uint32_t)(g * 16);
+        const uint32_t xo = (uint32_t)__shfl((int)aoff, tq * 16 + (lane >> 2), kWave) + (uint32_t)((lane & 3) * 16);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) xf[tq][ks] = *reinterpret_cast<const u32x4 *>(p.A + xo + ks * 64);
     }
+#pragma unroll
+    for (int tq = 0; tq < TQ; ++tq)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) xf[tq][ks] = lanes_4a_g_to_16g_a(xf[tq][ks], lane);
 
 #pragma unroll
     for (int tq = 0; tq < TQ; ++tq) {
