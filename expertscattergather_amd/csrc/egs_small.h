@@ -295,11 +295,11 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     }
     __syncthreads();
 
-    // block columns of this lane: X block at i0 + 4a (tile ci = column 4a + ci),
-    // Y block at j0 + 16*(a%4) + 4*(a/4) (tile cj), so that after the MFMA lane (a, g) holds,
-    // for row i = i0 + 4a + ci, the four consecutive columns j0 + 16r + 4g + cj
+    // block columns of this lane: X block at i0 + 4a (tile ci = column 4a + ci), Y block at j0 + 4a (tile cj):
+    // adjacent lanes fetch adjacent 8-byte pieces of a row, and after the MFMA lane (a, g) holds, for row
+    // i = i0 + 4a + ci, the four consecutive columns j0 + 16g + 4r + cj
     const uint32_t xcol = (uint32_t)min(i0 + a * 4, p.I - 4) * 2u;
-    const uint32_t ycol = (uint32_t)min(j0 + (a & 3) * 16 + (a >> 2) * 4, p.J - 4) * 2u;
+    const uint32_t ycol = (uint32_t)min(j0 + a * 4, p.J - 4) * 2u;
 
     f32x4 acc[4][4];            // [ci][cj]
 #pragma unroll
@@ -351,7 +351,7 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     for (int ci = 0; ci < 4; ++ci)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int i = a * 4 + ci, chunk = (r * 4 + g) ^ a;
+            const int i = a * 4 + ci, chunk = (g * 4 + r) ^ a;
             *reinterpret_cast<f32x4 *>(mine + i * 64 + chunk * 4) =
                 f32x4{acc[ci][0][r], acc[ci][1][r], acc[ci][2][r], acc[ci][3][r]};
         }
