@@ -408,7 +408,8 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
 {
     static size_t configured_plain = 64 * 1024, configured_dw = 64 * 1024;
     if (dw != nullptr) {
-        const size_t need = lds > (size_t)kDwSmallLdsBytes ? lds : (size_t)kDwSmallLdsBytes;
+        const size_t dw_lds = (size_t)kDwSmallLdsBytes * (kFusedThreads / kThreads);       // one 16 KB tile per wavefront
+        const size_t need = lds > dw_lds ? lds : dw_lds;
         if (need > configured_dw) {
             hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_dw_kernel<TT, W_NMAJOR, KS>,
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);

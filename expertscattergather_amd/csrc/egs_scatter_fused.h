@@ -207,8 +207,7 @@ __global__ __launch_bounds__(kFusedThreads) void scatter_fused_dw_kernel(Scatter
     if ((int)blockIdx.x < fused_blocks) {
         scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused_dw);
     } else {
-        if ((int)threadIdx.x >= kThreads) return;       // the weight gradient is written for four wavefronts
-        dw_small_body<TT>(q, (int)blockIdx.x - fused_blocks, reinterpret_cast<float *>(smem_fused_dw));
+        dw_small_body<TT, kFusedThreads / 64>(q, (int)blockIdx.x - fused_blocks, reinterpret_cast<float *>(smem_fused_dw));
     }
 }
 

@@ -260,10 +260,11 @@ constexpr int kDwSmallLdsBytes = 4 * 64 * 64 * 4;
 
 // Requirements: 2-byte elements, I % 8 == 0, J % 8 == 0, rows 16-byte aligned, spans < 4 GiB,
 // rows_per_split <= kDwSmallMaxRows.
-template <class TT>
+template <class TT, int NW = 4>
 __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int block, float *red)
 {
-    // red: kDwSmallLdsBytes of 16-byte aligned LDS, one 64 x 64 tile per wavefront
+    // NW wavefronts; red: NW * 16 KB of 16-byte aligned LDS (kDwSmallLdsBytes for four), one 64 x 64 tile per wavefront
+    constexpr int NT = NW * 64;
     uint32_t *xoff_lds = reinterpret_cast<uint32_t *>(red);              // reused before the reduction:
     uint32_t *yoff_lds = xoff_lds + kDwSmallMaxRows;                      //   row byte offsets, 0xFFFFFFFF = no row
 
@@ -280,7 +281,7 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     const int row_begin = s * p.rows_per_split;
     const int nrows = max(0, min(Me, row_begin + p.rows_per_split) - row_begin);
 
-    for (int r = tid; r < p.rows_per_split; r += kThreads) {
+    for (int r = tid; r < p.rows_per_split; r += NT) {
         uint32_t xo = 0xFFFFFFFFu, yo = 0;
         if (r < nrows) {
             const int m = row_begin + r;
@@ -337,8 +338,8 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     if (wave < nsteps) {
         Stage cur, nxt;
         load_stage(wave, cur);
-        for (int step = wave; step < nsteps; step += 4) {
-            if (step + 4 < nsteps) load_stage(step + 4, nxt);
+        for (int step = wave; step < nsteps; step += NW) {
+            if (step + NW < nsteps) load_stage(step + NW, nxt);
             consume(cur);
             cur = nxt;
         }
@@ -363,14 +364,14 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     // element-wise sum.
     const bool direct = (p.S == 1);
     const bool eji = p.dw_layout != 0;
-    for (int item = tid; item < 64 * 16; item += kThreads) {
+    for (int item = tid; item < 64 * 16; item += NT) {
         const int major = item >> 4, minor4 = (item & 15) * 4;      // major: i (EIJ) or j (EJI); minor: 4 x j or 4 x i
         f32x4 v;
         if (!eji) {
             const int phys = ((minor4 >> 2) ^ (major >> 2)) * 4;
             v = *reinterpret_cast<const f32x4 *>(red + major * 64 + phys);
 #pragma unroll
-            for (int w = 1; w < 4; ++w) {
+            for (int w = 1; w < NW; ++w) {
                 const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * 4096 + major * 64 + phys);
                 v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
             }
@@ -381,7 +382,7 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
                 const int at = i * 64 + (((major >> 2) ^ (i >> 2)) * 4) + (major & 3);
                 float acc1 = red[at];
 #pragma unroll
-                for (int w = 1; w < 4; ++w) acc1 += red[w * 4096 + at];
+                for (int w = 1; w < NW; ++w) acc1 += red[w * 4096 + at];
                 v[x] = acc1;
             }
         }
