@@ -104,6 +104,14 @@ def _workspace(dev: torch.device, nbytes: int):
     return buf.data_ptr(), buf.numel()
 
 
+def release_workspaces() -> None:
+    """Drop the cached scratch buffers (one per device and stream that has run a scatter or a backward).
+
+    They are re-created on demand; call this after a burst of work on short-lived streams, or
+    before measuring peak memory."""
+    _workspaces.clear()
+
+
 def _rows_source(X: torch.Tensor):
     """[B,T,I] tensor -> (tensor with unit inner stride, batch stride, token stride)."""
     if X.stride(2) != 1 and X.shape[2] > 1:

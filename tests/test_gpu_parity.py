@@ -384,3 +384,23 @@ def test_fp8_weight_gather_matches_dequantised_oracle():
     Y = hk.expert_gather_fp8w_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
     ref = O.gather_forward_fp8w(np64(case["X"]), Wq.view(torch.uint8).numpy(), scale.numpy(), case["Ind"].numpy())
     assert_close(Y, ref, torch.bfloat16, "fp8 weights large")
+
+
+def test_ops_pass_opcheck_and_router_output_feeds_the_kernels():
+    # registration of the four ops (schema, fake implementations, no hidden mutation), the counterpart of the
+    # reference's ~220 lines of torch.library glue (egs/triton_kernels.py:361-578)
+    from expertscattergather_amd.router import expert_choice_router
+    hk.create_kernels()
+    B, T, E, K, I, J = 2, 24, 3, 5, 32, 16
+    case = make_case(41, B, T, E, K, I, J, torch.float32)
+    logits = torch.randn(B, T, E, generator=torch.Generator().manual_seed(1))
+    Ind, _ = expert_choice_router(dev(logits), K, torch.int32)
+    X, Wg, Ws, Y, dOut = (dev(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut"))
+    ops = torch.ops.egs_amd
+    tests = ("test_schema", "test_faketensor")
+    torch.library.opcheck(ops.expert_gather_forward_call_fn.default, (X, Wg, Ind, torch.float32), test_utils=tests)
+    torch.library.opcheck(ops.expert_scatter_forward_call_fn.default, (Y, Ws, Ind, T, torch.float32), test_utils=tests)
+    torch.library.opcheck(ops.expert_gather_backward_call_fn.default, (X, Wg, Ind, Y, torch.float32), test_utils=tests)
+    torch.library.opcheck(ops.expert_scatter_backward_call_fn.default, (Y, Ws, Ind, dOut, torch.float32), test_utils=tests)
+    got = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    assert_close(got, O.gather_forward(np64(case["X"]), np64(case["Wg"]), Ind.cpu().numpy().astype("int64")), torch.float32, "router picks")

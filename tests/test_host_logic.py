@@ -96,3 +96,25 @@ def test_workloads_follow_the_benchmark_configurations():
     Wq, scale = wl.quantize_fp8_weights(torch.randn(3, 16, 8))
     assert Wq.dtype == torch.float8_e4m3fn and scale.shape == (3, 8)
     assert (Wq.float().abs().amax(dim=1) <= 448).all()
+
+
+def test_expert_choice_router_picks_top_k_tokens_per_expert():
+    import torch
+    from expertscattergather_amd.router import expert_choice_router
+    gen = torch.Generator().manual_seed(3)
+    B, T, E, K = 3, 17, 5, 4
+    logits = torch.randn(B, T, E, generator=gen)
+    Ind, scores = expert_choice_router(logits, K, torch.int16)
+    assert Ind.shape == (B, E, K) and Ind.dtype == torch.int16 and scores.shape == (B, E, K)
+    aff = torch.softmax(logits, -1)
+    for b in range(B):
+        for e in range(E):
+            order = sorted(range(T), key=lambda t: -float(aff[b, t, e]))[:K]
+            assert Ind[b, e].tolist() == order
+            assert len(set(Ind[b, e].tolist())) == K
+            assert torch.allclose(scores[b, e], aff[b, Ind[b, e].long(), e])
+    import pytest
+    with pytest.raises(ValueError):
+        expert_choice_router(torch.randn(1, 300, 2), 2, torch.uint8)      # ids up to 299 do not fit
+    with pytest.raises(ValueError):
+        expert_choice_router(logits, T + 1)
