@@ -341,6 +341,18 @@ __device__ __forceinline__ u32x4 lanes_4a_g_to_16g_a(const u32x4 &v, int lane)
     return r;
 }
 
+// The inverse move: lane 4 a + g receives what lane 16 g + a holds.  Results of an MFMA tile have the four
+// lanes g = 0..3 of row a holding four consecutive 16-byte pieces of that row; regrouped, adjacent lanes
+// store adjacent addresses (one 64-byte access per row instead of four 16-byte ones).
+__device__ __forceinline__ u32x4 lanes_16g_a_to_4a_g(const u32x4 &v, int lane)
+{
+    const int src = ((lane & 3) << 4 | (lane >> 2)) << 2;
+    u32x4 r;
+#pragma unroll
+    for (int x = 0; x < 4; ++x) r[x] = (uint32_t)__builtin_amdgcn_ds_bpermute(src, (int)v[x]);
+    return r;
+}
+
 // workgroup id -> (expert, tile): consecutive workgroup ids land on consecutive XCDs (8 per
 // device), so expert = 8*group + (id % 8) keeps all tiles of one expert on one XCD and its
 // weight tile in that XCD's L2.

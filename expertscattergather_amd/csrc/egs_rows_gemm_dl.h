@@ -44,14 +44,9 @@ __host__ __device__ constexpr int dl_smem_bytes_scatter(int BM, int BK, int NSTA
 // swizzle of the [reduction][column] tile: 32-byte units of a row are XORed with bits {0,1,3} of
 // the row number, which spreads the 16 rows one transpose read touches over all banks
 __device__ __forceinline__ int tr_swizzle(int row) { return (row & 3) | (((row >> 3) & 1) << 2); }
-// swizzle keys of the K-major tiles (XORed into the 16-byte chunk index of a row of CR chunks), chosen
-// so that the 16 lanes of one fragment read hit 16 different 16-byte bank groups.  The row side reads
-// 16 consecutive rows; the weight side reads the relabelled rows 16 c + 4 j + d (c, d = 0..3).
+// swizzle key of the K-major tiles (XORed into the 16-byte chunk index of a row of CR chunks), chosen so
+// that the 16 lanes of one fragment read (16 consecutive rows) hit 16 different 16-byte bank groups.
 template <int CR> __device__ __forceinline__ int kmajor_key_rows(int row) { return CR == 8 ? (row & 7) : ((row >> 2) & 3); }
-template <int CR> __device__ __forceinline__ int kmajor_key_relabelled(int row)
-{
-    return CR == 8 ? ((((row >> 4) & 3) << 1) | ((row >> 1) & 1)) : ((row >> 4) & 3);
-}
 
 template <class TT, int WES, int BM, int BK, int NSTAGE, bool GATHER, bool W_TRANS, int EPI>
 __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
@@ -136,7 +131,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
         if constexpr (!W_TRANS) {
             const int row = (wave * QL + jj) * (64 / CR) + lane / CR;
             const int n = n0 + row;
-            qv[jj] = n < N ? (uint32_t)n * (uint32_t)R * 2 + (((lane % CR) ^ kmajor_key_relabelled<CR>(row)) << 4) : kVoffInvalid;
+            qv[jj] = n < N ? (uint32_t)n * (uint32_t)R * 2 + (((lane % CR) ^ kmajor_key_rows<CR>(row)) << 4) : kVoffInvalid;
         } else if constexpr (W_FP8) {
             // bytes, [BK reduction rows][16 chunks]: a load covers 4 rows; lane l lands on row 4j + l/16, physical
             // chunk l%16; chunks are XORed with the low four bits of the row so that the 32 rows one transpose
@@ -177,8 +172,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
         m_at[ks] = (wave_m0 + a) * (BK * 2) + (((ks * 4 + g) ^ kmajor_key_rows<CR>(wave_m0 + a)) << 4);
-    // weight side, K-major: rows relabelled so that a lane ends up with 16 consecutive output columns,
-    //   row(j) = wave_n0 + 16 (a/4) + 4 j + a%4   (key does not depend on j)
+    // weight side, K-major: row(j) = wave_n0 + 16 j + a, read like the row side
     // weight side, [reduction][column]: lane supplies row 32 ks + 8 g + 4 h + a/4 and columns
     //   wave_n0 + 16 j + 4 (a%4) .. +3, so it receives column wave_n0 + 16 j + a   (fp8: row 32 ks + 8 g + a/2,
     //   bytes 8 (a%2) .. +7 of the 16-byte chunk of tile j)
@@ -188,8 +182,8 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             if constexpr (!W_TRANS) {
-                const int row = wave_n0 + (a >> 2) * 16 + (a & 3);
-                n_at[ks][h] = row * (BK * 2) + (((ks * 4 + g) ^ kmajor_key_relabelled<CR>(row)) << 4);
+                const int row = wave_n0 + a;                    // + 16 j: the key does not depend on j
+                n_at[ks][h] = row * (BK * 2) + (((ks * 4 + g) ^ kmajor_key_rows<CR>(row)) << 4);
             } else if constexpr (W_FP8) {
                 const int row = ks * 32 + g * 8 + (a >> 1);
                 n_at[ks][h] = row * 256 + (((wave_n0 >> 4) ^ (row & 15)) << 4) + (a & 1) * 8;
@@ -224,7 +218,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (!W_TRANS) {
-                    nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][0] + j * (4 * BK * 2));
+                    nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][0] + j * (16 * BK * 2));
                 } else if constexpr (W_FP8) {
                     u32x2 q8 = lds_read_tr8(tile_n + (n_at[ks][0] ^ (j << 4)));      // chunk wave_n0/16 + j, j < 4
                     nf[j] = fp8x8_to_bf16_chunk(q8[0], q8[1]);
@@ -243,29 +237,32 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
         if (++stage == NSTAGE) stage = 0;
     }
 
-    // ---------------- epilogue: 4 (transposed weights) or 16 (K-major weights) consecutive columns per lane and row
+    // ---------------- epilogue.  After the MFMAs lane (a, g) holds, for row 16 i + a, the four columns
+    // 16 j + 4 g .. + 3.  The values are regrouped across lanes first (lane 4 r + c takes piece c of row r),
+    // so that the four pieces of a row, 64 contiguous bytes of fp32 or 32 of a 16-bit type, leave from
+    // adjacent lanes as one access.
     constexpr int OES = (EPI == EPI_STORE_F32) ? 4 : 2;
+    const int srow = lane >> 2, sg = lane & 3;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        int64_t co = c_off[wave_m0 + i * 16 + a];
-        if (co < 0) continue;
+        const int64_t co = c_off[wave_m0 + i * 16 + srow];
         char *crow = p.C + co * OES;
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
-            int n = n0 + wave_n0 + (W_TRANS ? j * 16 + g * 4 : g * 16 + j * 4);
-            if (n >= N) continue;              // N % 8 == 0 and n % 4 == 0: the 4 columns are all in or all out
             f32x4 v = acc[i][j];
             if (p.w_scale != nullptr) {
+                const int nn = n0 + wave_n0 + j * 16 + g * 4;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] *= p.w_scale[(size_t)e * N + n + r];
+                for (int r = 0; r < 4; ++r) v[r] *= nn + r < N ? p.w_scale[(size_t)e * N + nn + r] : 0.f;
             }
+            const int n = n0 + wave_n0 + j * 16 + sg * 4;      // N % 8 == 0 and n % 4 == 0: the 4 columns are all in or all out
             if constexpr (OES == 4) {
-                *reinterpret_cast<f32x4 *>(crow + (size_t)n * 4) = v;
+                const u32x4 w = lanes_16g_a_to_4a_g(__builtin_bit_cast(u32x4, v), lane);
+                if (co >= 0 && n < N) *reinterpret_cast<u32x4 *>(crow + (size_t)n * 4) = w;
             } else {
-                u32x2 w;
-                w[0] = pack2<TT>(v[0], v[1]);
-                w[1] = pack2<TT>(v[2], v[3]);
-                *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = w;
+                u32x4 w = {pack2<TT>(v[0], v[1]), pack2<TT>(v[2], v[3]), 0u, 0u};
+                w = lanes_16g_a_to_4a_g(w, lane);
+                if (co >= 0 && n < N) *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = u32x2{w[0], w[1]};
             }
         }
     }
