@@ -203,14 +203,14 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
 #pragma unroll
         for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // fragment rows.  Without SWAP the weight side supplies the accumulator's row axis and its
-    // rows are relabelled so that one lane ends up with 4*TN consecutive output columns.
+    // fragment rows.  Without SWAP the weight side supplies the accumulator's row axis: lane (a, g) ends up
+    // with columns 16 j + 4 g .. + 3 of row 16 i + a.
     int mrow_l[TM], nrow_l[TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i) mrow_l[i] = wave_m0 + i * 16 + a;
 #pragma unroll
     for (int j = 0; j < TN; ++j)
-        nrow_l[j] = SWAP ? wave_n0 + j * 16 + a : wave_n0 + (a >> 2) * (4 * TN) + j * 4 + (a & 3);
+        nrow_l[j] = wave_n0 + j * 16 + a;
 
     const int nk = (R + BK - 1) / BK;
     for (int kt = 0; kt < nk; ++kt) {
@@ -240,23 +240,27 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
 
     // ---------------- epilogue
     if constexpr (!SWAP) {
+        // results are regrouped across lanes first (lane 4 r + c takes piece c of row r), so that the four
+        // pieces of a row leave from adjacent lanes as one contiguous access
         constexpr int OES = (EPI == EPI_STORE_F32) ? 4 : ES;
         const bool c_vec = p.c_vec != 0;
+        const int srow = lane >> 2, sg = lane & 3;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            int64_t co = c_off[wave_m0 + i * 16 + a];
-            if (co < 0) continue;
-            char *crow = p.C + co * OES;
+            const int64_t co = c_off[wave_m0 + i * 16 + srow];
+            char *crow = p.C + (co < 0 ? 0 : co) * OES;
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                int n = n0 + wave_n0 + g * (4 * TN) + j * 4;
-                if (n >= N) continue;
                 f32x4 v = acc[i][j];
                 if (p.w_scale != nullptr) {
+                    const int nn = n0 + wave_n0 + j * 16 + g * 4;
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (n + r < N) v[r] *= p.w_scale[(size_t)e * N + n + r];
+                        if (nn + r < N) v[r] *= p.w_scale[(size_t)e * N + nn + r];
                 }
+                v = __builtin_bit_cast(f32x4, lanes_16g_a_to_4a_g(__builtin_bit_cast(u32x4, v), lane));
+                const int n = n0 + wave_n0 + j * 16 + sg * 4;
+                if (co < 0 || n >= N) continue;
                 if (c_vec && n + 4 <= N) {
                     if constexpr (OES == 4) {
                         *reinterpret_cast<f32x4 *>(crow + (size_t)n * 4) = v;
