@@ -30,7 +30,8 @@ MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
 # Counters cannot be read from inside this process, so the figure is the recorded one.
-MEASURED_TRAFFIC_BYTES = {("C2", "gather_gemm"): 17349000}
+MEASURED_TRAFFIC_BYTES = {("C2", "gather_gemm"): 17349000,        # profiles/rows_small_gather_c2_traffic.md
+                          ("C3", "gather_gemm"): 693100000}       # profiles/rows_gemm_dl_gather_c3_counters.md
 
 
 def parse_args():
