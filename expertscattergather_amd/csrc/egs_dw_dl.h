@@ -18,6 +18,7 @@
 #pragma once
 #include "egs_dw.h"
 #include "egs_rows_gemm_dl.h"
+#include "egs_small.h"
 
 namespace egs {
 
@@ -194,8 +195,14 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
             if (j >= p.J) continue;                 // J % 8 == 0: the four columns are all in or all out
             f32x4 v = acc[x][y];
             if (!direct) {
-                float *dst = p.part + (((size_t)s * p.E + e) * p.I + i) * p.J + j;
-                *reinterpret_cast<f32x4 *>(dst) = v;            // workspace base is 256-byte aligned, J % 4 == 0
+                // partial sums already in the layout of the output, so that the second pass is a plain sum
+                if (p.dw_layout == 0) {
+                    float *dst = p.part + (((size_t)s * p.E + e) * p.I + i) * p.J + j;
+                    *reinterpret_cast<f32x4 *>(dst) = v;        // workspace base is 256-byte aligned, J % 4 == 0
+                } else {                                        // [E,J,I]: 16 lanes cover 16 consecutive i
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) p.part[(((size_t)s * p.E + e) * p.J + (j + r)) * p.I + i] = v[r];
+                }
             } else if (p.dw_layout == 0) {                      // [E,I,J]
                 size_t at = ((size_t)e * p.I + i) * p.J + j;
                 if (p.out_dtype == 0) {

@@ -43,10 +43,10 @@ int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *
             else hipLaunchKernelGGL((dw_dl_kernel<ElemBF16, 128>), dim3((unsigned)grid), dim3(kDlThreads), 0, s, q);
         }
         EGS_CHECK_LAUNCH("dw_dl_kernel");
-        if (pl.b_S > 1) {
-            hipLaunchKernelGGL(dw_reduce_kernel, dim3(grid_1d(w_elems, 4096)), dim3(kThreads), 0, s, (const float *)workspace,
-                               (char *)dW, pl.b_S, d->E, d->I, d->J, out_dtype, dw_layout);
-            EGS_CHECK_LAUNCH("dw_reduce_kernel");
+        if (pl.b_S > 1) {       // partials are in the output's layout, I % 8 == 0 and J % 8 == 0: vectorised plain sum
+            hipLaunchKernelGGL(dw_reduce4_kernel, dim3(grid_1d(w_elems / 4, 4096)), dim3(kThreads), 0, s,
+                               (const float *)workspace, (char *)dW, pl.b_S, w_elems / 4, out_dtype);
+            EGS_CHECK_LAUNCH("dw_reduce4_kernel");
         }
         return EGS_OK;
     }
