@@ -404,3 +404,41 @@ def test_ops_pass_opcheck_and_router_output_feeds_the_kernels():
     torch.library.opcheck(ops.expert_scatter_backward_call_fn.default, (Y, Ws, Ind, dOut, torch.float32), test_utils=tests)
     got = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
     assert_close(got, O.gather_forward(np64(case["X"]), np64(case["Wg"]), Ind.cpu().numpy().astype("int64")), torch.float32, "router picks")
+
+
+@pytest.mark.parametrize("shape", [(8, 64, 8, 16, 128, 64), (2, 300, 4, 200, 256, 192)], ids=["small-experts", "large-tiles"])
+def test_graph_replays_match_eager_results(shape):
+    # the whole forward+backward sequence captured once and replayed with other work in between: every replay
+    # must reproduce the eager results bit for bit (scratch is cleared by kernels, nothing depends on capture-time state)
+    B, T, E, K, I, J = shape
+    case = make_case(51, B, T, E, K, I, J, torch.bfloat16)
+    X, Wg, Ws, dOut, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "dOut", "Ind"))
+    hk.set_scatter_mode("deterministic")
+
+    def step():
+        Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+        dY, dWs = hk.expert_scatter_backward_call(Y, Ws, Ind, dOut, torch.float32)
+        dX, dWg = hk.expert_gather_backward_call(X, Wg, Ind, dY, torch.float32)
+        return Y, out, dX, dWg, dWs
+
+    eager = [t.clone() for t in step()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = step()
+    for rep in range(4):
+        for t in outs:
+            t.fill_(float("nan"))                   # stale results must not survive a replay
+        junk = torch.randn(1 << 18, device=DEV).sum()      # unrelated eager work between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, ref in zip(("Y", "out", "dX", "dWg", "dWs"), outs, eager):
+            assert torch.equal(got, ref), f"replay {rep}: {name} differs from the eager result"
+        del junk
