@@ -407,7 +407,9 @@ template <class TT, bool W_NMAJOR, int KS>
 int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
 {
     static size_t configured_plain = 64 * 1024, configured_dw = 64 * 1024;
+    if constexpr (TT::ES != 2) dw = nullptr;            // the small weight gradient exists for 16-bit types only
     if (dw != nullptr) {
+      if constexpr (TT::ES == 2) {
         const size_t dw_lds = (size_t)kDwSmallLdsBytes * (kFusedThreads / kThreads);       // one 16 KB tile per wavefront
         const size_t need = lds > dw_lds ? lds : dw_lds;
         if (need > configured_dw) {
@@ -419,6 +421,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
         hipLaunchKernelGGL((scatter_fused_dw_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dw->blocks), dim3(kFusedThreads), need, s, p,
                            dw->q, blocks);
         dw->done = true;
+      }
     } else {
         if (lds > configured_plain) {
             hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_kernel<TT, W_NMAJOR, KS>,
@@ -435,9 +438,9 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
 template <class TT, bool W_NMAJOR>
 int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
 {
-    switch (R) {
-    case 32: return launch_scatter_fused_one<TT, W_NMAJOR, 1>(p, lds, blocks, dw, s);
-    case 64: return launch_scatter_fused_one<TT, W_NMAJOR, 2>(p, lds, blocks, dw, s);
+    switch (R / (4 * TT::VEC)) {        // MFMA steps of four 16-byte chunks
+    case 1: return launch_scatter_fused_one<TT, W_NMAJOR, 1>(p, lds, blocks, dw, s);
+    case 2: return launch_scatter_fused_one<TT, W_NMAJOR, 2>(p, lds, blocks, dw, s);
     default: return launch_scatter_fused_one<TT, W_NMAJOR, 4>(p, lds, blocks, dw, s);
     }
 }
@@ -450,12 +453,13 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     used = false;
     const int R = d->J, N = d->I;
     const int64_t NP = (int64_t)d->E * d->K;
-    if (g_force_generic || act_dtype == EGS_F32 || !(R == 32 || R == 64 || R == 128)) return EGS_OK;
+    if (g_force_generic || !(R == 32 || R == 64 || (R == 128 && act_dtype != EGS_F32))) return EGS_OK;
+    const int ES = elem_size(act_dtype);
     if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 1024 || d->T < 1 || d->B < 1) return EGS_OK;
     const size_t lds = scatter_fused_lds(d->T, (int)NP);
     if (lds > 156 * 1024) return EGS_OK;
-    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 8)) return EGS_OK;
-    if ((uint64_t)d->B * NP * R * 2 > kSpan32 || (uint64_t)d->E * R * N * 2 > kSpan32) return EGS_OK;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 16)) return EGS_OK;
+    if ((uint64_t)d->B * NP * R * ES > kSpan32 || (uint64_t)d->E * R * N * ES > kSpan32) return EGS_OK;
     const int slices = N / kFusedCols;
     const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
     if (blocks > INT32_MAX / 2 || (int64_t)d->B * slices < 8) return EGS_OK;        // too few workgroups to be worth it
@@ -469,6 +473,9 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
     used = true;
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
+    if (act_dtype == EGS_F32)
+        return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, s)
+                      : launch_scatter_fused_ks<ElemF32, false>(p, R, lds, (int)blocks, nullptr, s);
     if (act_dtype == EGS_F16)
         return nmajor ? launch_scatter_fused_ks<ElemF16, true>(p, R, lds, (int)blocks, dw, s)
                       : launch_scatter_fused_ks<ElemF16, false>(p, R, lds, (int)blocks, dw, s);

@@ -16,7 +16,8 @@
 // reference's default shape.  Bitwise reproducible (fixed order), no atomics.
 //
 // Fits when a batch element's picks (E*K <= 1024) times 128 bytes, the table and the sort's
-// histograms fit in LDS; 16-bit elements, reduction 32/64/128, output columns a multiple of 32.
+// histograms fit in LDS; 16-bit elements with reduction 32/64/128 or fp32 with reduction 32/64, output
+// columns a multiple of 32.
 //
 // Replaces the reference's expert_scatter_kernel (egs/triton_kernels.py:156-247), which adds every
 // output element with a global atomic.
@@ -31,7 +32,7 @@ constexpr int kFusedCols = 32;          // output columns per workgroup
 constexpr int kFusedThreads = 512;      // 8 wavefronts: enough units in flight to cover the memory latency in two rounds
 
 struct ScatterFusedParams {
-    const char *A;          // [B,E,K,R] dense rows, 16-bit
+    const char *A;          // [B,E,K,R] dense rows
     const char *W;          // [E,R,N] (W_NMAJOR) or [E,N,R]
     const void *Ind;        // [B,E,K]
     char *out;              // [B,T,N] element type
@@ -50,8 +51,9 @@ __host__ __device__ inline size_t scatter_fused_lds(int T, int NP)
 template <class TT, bool W_NMAJOR, int KS>
 __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, const int block, char *smem)
 {
-    static_assert(TT::ES == 2, "16-bit element types");
-    constexpr int R = 32 * KS;
+    // KS = reduction length in MFMA steps of four 16-byte chunks: 32 elements of a 16-bit type, 16 of fp32
+    constexpr int ES = TT::ES, VEC = TT::VEC;
+    constexpr int R = 4 * VEC * KS;
     constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 32-pick) units in flight per wavefront
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int a = lane & 15, g = lane >> 4;
@@ -75,7 +77,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     const int units = E * KT2;
     struct Unit { u32x4 y[2][KS]; u32x4 w[2 * KS]; };
     Unit buf[kFusedDepth];
-    const uint32_t a_base_b = (uint32_t)b * (uint32_t)NP * R * 2;
+    const uint32_t a_base_b = (uint32_t)b * (uint32_t)NP * R * ES;
     auto load_unit = [&](Unit &u, int unit) {
         unit = min(unit, units - 1);                    // unconditional loads; surplus units are not stored
         const int e = unit / KT2, rp = unit - e * KT2;
@@ -83,26 +85,35 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
         for (int h = 0; h < 2; ++h) {
             // coalesced: lanes 4r .. 4r+3 fetch four consecutive chunks of row r; transposed to operand order at use
             const int k = min(rp * 32 + h * 16 + (lane >> 2), K - 1);
-            const char *yrow = p.A + a_base_b + (uint32_t)((e * K + k) * R * 2);
+            const char *yrow = p.A + a_base_b + (uint32_t)((e * K + k) * R * ES);
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) u.y[h][ks] = *reinterpret_cast<const u32x4 *>(yrow + (ks * 32 + (lane & 3) * 8) * 2);
+            for (int ks = 0; ks < KS; ++ks) u.y[h][ks] = *reinterpret_cast<const u32x4 *>(yrow + (ks * 4 + (lane & 3)) * 16);
         }
         if constexpr (!W_NMAJOR) {
             // [E,N,R]: the lane's output column is a row of W
 #pragma unroll
             for (int ct = 0; ct < 2; ++ct) {
-                const char *wrow = p.W + ((size_t)e * N + c0 + ct * 16 + (lane >> 2)) * (R * 2);
+                const char *wrow = p.W + ((size_t)e * N + c0 + ct * 16 + (lane >> 2)) * (R * ES);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) u.w[ct * KS + ks] = *reinterpret_cast<const u32x4 *>(wrow + (ks * 32 + (lane & 3) * 8) * 2);
+                for (int ks = 0; ks < KS; ++ks) u.w[ct * KS + ks] = *reinterpret_cast<const u32x4 *>(wrow + (ks * 4 + (lane & 3)) * 16);
             }
         } else {
-            // [E,R,N]: 8 (reduction) x 2 (columns 2a, 2a+1) blocks, transposed in registers below; raw rows kept here
+            // [E,R,N]: VEC (reduction) x 2 (columns 2a, 2a+1) blocks, transposed in registers below; raw rows kept here
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                const char *wblk = p.W + (((size_t)e * R + ks * 32 + g * 8) * N + c0 + 2 * a) * 2;
+                const char *wblk = p.W + (((size_t)e * R + ks * 4 * VEC + g * VEC) * N + c0 + 2 * a) * ES;
+                if constexpr (ES == 2) {
 #pragma unroll
-                for (int x = 0; x < 8; ++x)
-                    u.w[ks * 2 + (x >> 2)][x & 3] = *reinterpret_cast<const uint32_t *>(wblk + (size_t)x * N * 2);
+                    for (int x = 0; x < 8; ++x)
+                        u.w[ks * 2 + (x >> 2)][x & 3] = *reinterpret_cast<const uint32_t *>(wblk + (size_t)x * N * 2);
+                } else {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const u32x2 two = *reinterpret_cast<const u32x2 *>(wblk + (size_t)x * N * 4);
+                        u.w[ks * 2 + (x >> 1)][(x & 1) * 2] = two[0];
+                        u.w[ks * 2 + (x >> 1)][(x & 1) * 2 + 1] = two[1];
+                    }
+                }
             }
         }
     };
@@ -117,12 +128,18 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
             u32x4 wf[2];
             if constexpr (!W_NMAJOR) {
                 wf[0] = lanes_4a_g_to_16g_a(u.w[ks], lane); wf[1] = lanes_4a_g_to_16g_a(u.w[KS + ks], lane);
-            } else {
+            } else if constexpr (ES == 2) {
 #pragma unroll
                 for (int pp = 0; pp < 4; ++pp) {
                     const uint32_t lo = u.w[ks * 2 + (pp >> 1)][(pp & 1) * 2], hi = u.w[ks * 2 + (pp >> 1)][(pp & 1) * 2 + 1];
                     wf[0][pp] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);     // column 2a   of rows 2pp, 2pp+1
                     wf[1][pp] = __builtin_amdgcn_perm(hi, lo, 0x07060302u);     // column 2a+1
+                }
+            } else {
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {                                   // row x of the block: columns 2a, 2a+1
+                    wf[0][x] = u.w[ks * 2 + (x >> 1)][(x & 1) * 2];
+                    wf[1][x] = u.w[ks * 2 + (x >> 1)][(x & 1) * 2 + 1];
                 }
             }
 #pragma unroll
@@ -184,10 +201,15 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
             for (int x = 0; x < 4; ++x)
                 if (s + x < s1) sum += v[x];
         }
-        u32x2 w;
-        w[0] = pack2<TT>(sum[0], sum[1]);
-        w[1] = pack2<TT>(sum[2], sum[3]);
-        *reinterpret_cast<u32x2 *>(p.out + (((size_t)b * T + t) * N + c0 + cc * 4) * 2) = w;
+        char *dst = p.out + (((size_t)b * T + t) * N + c0 + cc * 4) * ES;
+        if constexpr (ES == 4) {
+            *reinterpret_cast<f32x4 *>(dst) = sum;
+        } else {
+            u32x2 w;
+            w[0] = pack2<TT>(sum[0], sum[1]);
+            w[1] = pack2<TT>(sum[2], sum[3]);
+            *reinterpret_cast<u32x2 *>(dst) = w;
+        }
     }
 }
 
