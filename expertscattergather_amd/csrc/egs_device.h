@@ -254,11 +254,12 @@ __device__ __forceinline__ void direct_load16(u32x4 rsrc, uint32_t voff, uint32_
                  : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                  : "memory", "m0");
 }
-// Wait until at most N of this wavefront's vector-memory loads are outstanding (N < 16).
+// Wait until at most N of this wavefront's vector-memory operations are outstanding (N < 64; loads and
+// stores complete in issue order as far as this counter is concerned).
 template <int N> __device__ __forceinline__ void wait_vmem()
 {
-    static_assert(N >= 0 && N < 16, "immediate range");
-    __builtin_amdgcn_s_waitcnt(0x0f70 | N);
+    static_assert(N >= 0 && N < 64, "immediate range");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 // LDS transpose read: the 16 lanes of a group each point at 4 consecutive 16-bit elements of a
 // row (lanes 4k..4k+3 cover 16 columns of row k, k = 0..3); lane n receives column n of those four

@@ -237,32 +237,89 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
         if (++stage == NSTAGE) stage = 0;
     }
 
-    // ---------------- epilogue.  After the MFMAs lane (a, g) holds, for row 16 i + a, the four columns
-    // 16 j + 4 g .. + 3.  The values are regrouped across lanes first (lane 4 r + c takes piece c of row r),
-    // so that the four pieces of a row, 64 contiguous bytes of fp32 or 32 of a 16-bit type, leave from
-    // adjacent lanes as one access.
     constexpr int OES = (EPI == EPI_STORE_F32) ? 4 : 2;
-    const int srow = lane >> 2, sg = lane & 3;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int64_t co = c_off[wave_m0 + i * 16 + srow];
-        char *crow = p.C + co * OES;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            f32x4 v = acc[i][j];
-            if (p.w_scale != nullptr) {
-                const int nn = n0 + wave_n0 + j * 16 + g * 4;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] *= nn + r < N ? p.w_scale[(size_t)e * N + nn + r] : 0.f;
+    if constexpr (OES == 4) {
+        // fp32 product rows: measured slightly faster straight from registers than through LDS
+        // ---------------- epilogue.  After the MFMAs lane (a, g) holds, for row 16 i + a, the four columns
+        // 16 j + 4 g .. + 3.  The values are regrouped across lanes first (lane 4 r + c takes piece c of row r),
+        // so that the four pieces of a row, 64 contiguous bytes of fp32 or 32 of a 16-bit type, leave from
+        // adjacent lanes as one access.
+        const int srow = lane >> 2, sg = lane & 3;
+    #pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int64_t co = c_off[wave_m0 + i * 16 + srow];
+            char *crow = p.C + co * OES;
+    #pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                f32x4 v = acc[i][j];
+                if (p.w_scale != nullptr) {
+                    const int nn = n0 + wave_n0 + j * 16 + g * 4;
+    #pragma unroll
+                    for (int r = 0; r < 4; ++r) v[r] *= nn + r < N ? p.w_scale[(size_t)e * N + nn + r] : 0.f;
+                }
+                const int n = n0 + wave_n0 + j * 16 + sg * 4;      // N % 8 == 0 and n % 4 == 0: the 4 columns are all in or all out
+                if constexpr (OES == 4) {
+                    const u32x4 w = lanes_16g_a_to_4a_g(__builtin_bit_cast(u32x4, v), lane);
+                    if (co >= 0 && n < N) *reinterpret_cast<u32x4 *>(crow + (size_t)n * 4) = w;
+                } else {
+                    u32x4 w = {pack2<TT>(v[0], v[1]), pack2<TT>(v[2], v[3]), 0u, 0u};
+                    w = lanes_16g_a_to_4a_g(w, lane);
+                    if (co >= 0 && n < N) *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = u32x2{w[0], w[1]};
+                }
             }
-            const int n = n0 + wave_n0 + j * 16 + sg * 4;      // N % 8 == 0 and n % 4 == 0: the 4 columns are all in or all out
-            if constexpr (OES == 4) {
-                const u32x4 w = lanes_16g_a_to_4a_g(__builtin_bit_cast(u32x4, v), lane);
-                if (co >= 0 && n < N) *reinterpret_cast<u32x4 *>(crow + (size_t)n * 4) = w;
-            } else {
-                u32x4 w = {pack2<TT>(v[0], v[1]), pack2<TT>(v[2], v[3]), 0u, 0u};
-                w = lanes_16g_a_to_4a_g(w, lane);
-                if (co >= 0 && n < N) *reinterpret_cast<u32x2 *>(crow + (size_t)n * 2) = u32x2{w[0], w[1]};
+        }
+    } else {
+        // ---------------- epilogue.  After the MFMAs lane (a, g) holds, for row 16 i + a, the four columns
+        // 16 j + 4 g .. + 3: pieces of 16 rows per store.  The tile goes through LDS instead (the slab stages are
+        // free now), 128 rows of fp32 (or all 256 rows of a 16-bit type) at a time, and leaves as whole row
+        // segments: one store instruction writes 1 KB of one row (fp32) or 512 bytes of each of two rows, which
+        // is what the write path wants (product rows are the largest stream of the scatter: 1 GB at C3).
+        // LDS row = 256 columns; its 16-byte chunks are XORed with the low four row bits so that the 16 lanes
+        // of a fragment (16 rows, same chunk) spread over the banks.
+        constexpr int ROW_BYTES = BN * OES;                 // 1024 or 512
+        constexpr int HALVES = (BM * ROW_BYTES) / (NSTAGE * STAGE) > 1 ? 2 : ((BM * ROW_BYTES > NSTAGE * STAGE) ? 2 : 1);
+        constexpr int ROWS_PER_PASS = BM / HALVES;
+        static_assert(ROWS_PER_PASS * ROW_BYTES <= NSTAGE * STAGE, "staging tile fits the slab stages");
+        static_assert(HALVES == 1 || BM == 256, "two passes split the two wavefront rows of a 256-row tile");
+        constexpr int CPR = ROW_BYTES / 16;                  // chunks per staged row: 64 or 32
+    #pragma unroll 1
+        for (int half = 0; half < HALVES; ++half) {
+            __syncthreads();                                // stages (or the previous pass) no longer being read
+            if (HALVES == 1 || (wave >> 2) == half) {
+                const int row0 = (HALVES == 1 ? wave_m0 : 0) + a;
+    #pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int row = row0 + i * 16;
+    #pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        f32x4 v = acc[i][j];
+                        const int col = wave_n0 + j * 16 + g * 4;
+                        if (p.w_scale != nullptr) {
+    #pragma unroll
+                            for (int r = 0; r < 4; ++r) v[r] *= n0 + col + r < N ? p.w_scale[(size_t)e * N + n0 + col + r] : 0.f;
+                        }
+                        if constexpr (OES == 4) {
+                            const int chunk = (col >> 2) ^ (row & 15);
+                            *reinterpret_cast<f32x4 *>(smem + row * ROW_BYTES + chunk * 16) = v;
+                        } else {
+                            const int chunk = (col >> 3) ^ (row & 15);
+                            u32x2 w = {pack2<TT>(v[0], v[1]), pack2<TT>(v[2], v[3])};
+                            *reinterpret_cast<u32x2 *>(smem + row * ROW_BYTES + chunk * 16 + (col & 4) * 2) = w;
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            // every wavefront writes out its share of the staged rows, whole row segments per instruction
+            constexpr int LANES_PER_ROW = CPR;               // 64 (one row per instruction) or 32 (two rows)
+            constexpr int ROWS_PER_INSTR = 64 / LANES_PER_ROW;
+            const int lrow = lane / LANES_PER_ROW, lchunk = lane % LANES_PER_ROW;
+            const int n_here = n0 + lchunk * (16 / OES);
+            for (int r0 = wave * ROWS_PER_INSTR; r0 < ROWS_PER_PASS; r0 += NW * ROWS_PER_INSTR) {
+                const int row = r0 + lrow;
+                const int64_t co = c_off[half * ROWS_PER_PASS + row];
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + row * ROW_BYTES + ((lchunk ^ (row & 15)) << 4));
+                if (co >= 0 && n_here < N) *reinterpret_cast<u32x4 *>(p.C + co * OES + (size_t)n_here * OES) = v;
             }
         }
     }

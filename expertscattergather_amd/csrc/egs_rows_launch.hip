@@ -36,7 +36,7 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
             const bool dl = !g_force_generic && p.R % 64 == 0 && p.N % (WES == 1 ? 16 : 8) == 0 && p.a_vec && p.w_vec &&
                             p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && (WES == 1 || p.w_scale == nullptr) &&
                             (WES == 2 || aligned_to(p.W, 16)) &&
-                            (EPI == EPI_STORE_F32 ? aligned_to(p.C, 16) : aligned_to(p.C, 8));
+                            aligned_to(p.C, 16);
             if constexpr (WES == 2 || W_TRANS) {
                 if (dl) {
                     const size_t smem = GATHER ? 0 : (size_t)dl_smem_bytes_scatter(256, 64, 2);

@@ -31,6 +31,8 @@ SHAPES = [
     (3, 300, 5, 200, 192, 256),   # large products: 256 x 256 tiles, ragged last row tile, 192 of 256 columns
     (2, 128, 9, 260, 128, 200),   # large gather with half a 16-column tile at the edge
     (2, 200, 3, 128, 256, 72),    # large weight gradient without splits, 72 of 128 columns
+    (3, 100, 5, 200, 256, 128),   # large scatter products with a short reduction (128), ragged last row tile
+    (2, 80, 3, 260, 512, 256),    # the same with reduction 256 and two column tiles
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
