@@ -85,8 +85,32 @@ def _require_gpu(*tensors: torch.Tensor) -> torch.device:
     return dev
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream_ptr(dev: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(dev.index)
     return torch.cuda.current_stream(dev).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev: torch.device):
+    """Context that makes `dev` the current HIP device (the library launches on the current device);
+    nothing to do, and nothing paid, when it already is."""
+    if dev.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(dev)
 
 
 _workspaces: dict = {}
@@ -161,7 +185,7 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     W = W.contiguous(); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
                                                   ld_b, ld_t, dt, _ind_type_id(Ind), _stream_ptr(dev))
     _abi.check(rc, "expert_gather_forward_call")
@@ -180,7 +204,7 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     grad_W = torch.empty((E, I, J), device=dev, dtype=W.dtype)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt))
         rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
                                                    grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
@@ -201,7 +225,7 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     out = torch.empty((B, T, I), device=dev, dtype=Y.dtype)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt))
         rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
                                                    ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
@@ -220,7 +244,7 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
     grad_Y = torch.empty((B, E, K, J), device=dev, dtype=Y.dtype)
     grad_W = torch.empty((E, J, I), device=dev, dtype=W.dtype)
     d = _abi.Dims(B, T, E, K, I, J)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, d, dt))
         rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
                                                     grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
@@ -339,7 +363,7 @@ def expert_gather_fp8w_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.T
     Wq = Wq.contiguous(); scale = scale.contiguous(); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _abi.lib().egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), scale.data_ptr(), d,
                                         ld_b, ld_t, _abi.BF16, _abi.FP8_E4M3, _ind_type_id(Ind), _abi.W_EIJ,
                                         _stream_ptr(dev))
@@ -352,7 +376,7 @@ def validate_indices(Ind: torch.Tensor, T: int) -> int:
     dev = _require_gpu(Ind)
     Ind = Ind.contiguous()
     bad = torch.zeros(1, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         rc = _abi.lib().egs_validate_indices(Ind.data_ptr(), _ind_type_id(Ind), Ind.numel(), int(T), bad.data_ptr(),
                                              _stream_ptr(dev))
     _abi.check(rc, "validate_indices")
