@@ -1,8 +1,8 @@
 // The rows x weight product of egs_rows_gemm.h for large, well-formed 16-bit shapes, built around
 // what gfx950 adds for this: 16-byte direct global->LDS loads and LDS transpose reads.
 //
-//   * BM x 256 output tile (BM = 128 or 256), BK-deep slabs (32 or 64), BM/128 x 4 wavefronts, each
-//     128 x 64 of the tile.
+//   * BM x BN output tile (BM = 128 or 256, BN = 256, or 128 for outputs narrower than 192 columns),
+//     BK-deep slabs (32 or 64), BM/128 x BN/64 wavefronts, each 128 x 64 of the tile.
 //   * Both operand slabs travel HBM/L2 -> LDS without touching registers (one buffer load per
 //     1 KB of a slab), NSTAGE - 1 slabs in flight: the loads of slab k + NSTAGE - 1 are issued
 //     right after the barrier that publishes slab k and land while the MFMAs run.  One barrier
@@ -29,17 +29,19 @@
 
 namespace egs {
 
-constexpr int kDlBN = 256;
-
 // LDS bytes of one workgroup: slab stages, then the row tables (4 + 8 bytes per tile row)
-__host__ __device__ constexpr int dl_stage_bytes(int BM, int BK) { return (BM + kDlBN) * BK * 2; }
-__host__ __device__ constexpr int dl_smem_bytes(int BM, int BK, int NSTAGE) { return NSTAGE * dl_stage_bytes(BM, BK) + BM * 12; }
+__host__ __device__ constexpr int dl_stage_bytes(int BM, int BN, int BK) { return (BM + BN) * BK * 2; }
+__host__ __device__ constexpr int dl_smem_bytes(int BM, int BN, int BK, int NSTAGE)
+{
+    return NSTAGE * dl_stage_bytes(BM, BN, BK) + BM * 12;
+}
 // the scatter variants of the one-workgroup-per-CU shape reserve more, so that the routing-table
 // workgroups riding along have room for eight wavefronts' histograms at T = 4096
-__host__ __device__ constexpr int dl_smem_bytes_scatter(int BM, int BK, int NSTAGE)
+__host__ __device__ constexpr int dl_smem_bytes_scatter(int BM, int BN, int BK, int NSTAGE)
 {
-    return BM == 256 ? 150 * 1024 : dl_smem_bytes(BM, BK, NSTAGE);
+    return BM == 256 && BN == 256 ? 150 * 1024 : dl_smem_bytes(BM, BN, BK, NSTAGE);
 }
+__host__ __device__ constexpr int dl_threads(int BM, int BN) { return (BM / 128) * (BN / 64) * 64; }
 
 // swizzle of the [reduction][column] tile: 32-byte units of a row are XORed with bits {0,1,3} of
 // the row number, which spreads the 16 rows one transpose read touches over all banks
@@ -48,25 +50,29 @@ __device__ __forceinline__ int tr_swizzle(int row) { return (row & 3) | (((row >
 // that the 16 lanes of one fragment read (16 consecutive rows) hit 16 different 16-byte bank groups.
 template <int CR> __device__ __forceinline__ int kmajor_key_rows(int row) { return CR == 8 ? (row & 7) : ((row >> 2) & 3); }
 
-template <class TT, int WES, int BM, int BK, int NSTAGE, bool GATHER, bool W_TRANS, int EPI>
-__global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
+template <class TT, int WES, int BM, int BN, int BK, int NSTAGE, bool GATHER, bool W_TRANS, int EPI>
+__global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGemmParams p)
 {
     static_assert(TT::ES == 2, "16-bit element types");
     static_assert(EPI == EPI_STORE || EPI == EPI_STORE_F32, "plain stores only");
     static_assert(WES == 2 || (WES == 1 && W_TRANS && TT::ID == 2), "fp8 weights: [reduction][column] layout, widened to bf16");
-    static_assert((BM == 128 || BM == 256) && (BK == 32 || BK == 64) && (NSTAGE == 2 || NSTAGE == 3), "tile shapes");
+    static_assert((BM == 128 || BM == 256) && (BN == 128 || BN == 256) && (BK == 32 || BK == 64) &&
+                  (NSTAGE == 2 || NSTAGE == 3), "tile shapes");
     constexpr bool W_FP8 = (WES == 1);
-    constexpr int BN = kDlBN;
-    constexpr int NT = BM * 2, NW = NT / 64;             // BM/128 x 4 wavefronts
+    static_assert(!W_FP8 || BN == 256, "the fp8 tile layout is written for 256-byte rows");
+    constexpr int WN = BN / 64;                          // wavefront columns
+    constexpr int NT = dl_threads(BM, BN), NW = NT / 64; // BM/128 x BN/64 wavefronts
     constexpr int TM = 8, TN = 4;                        // 16 x 16 tiles per wavefront: 128 x 64
     constexpr int KSTEPS = BK / 32;
     constexpr int CR = BK / 8;                           // 16-byte chunks per K-major row
-    constexpr int P_BYTES = BM * BK * 2, STAGE = dl_stage_bytes(BM, BK);
+    constexpr int P_BYTES = BM * BK * 2, STAGE = dl_stage_bytes(BM, BN, BK);
     constexpr int PL = BM * CR / 64 / NW;                // loads per wavefront and slab: row side,
-    constexpr int QL = W_FP8 ? BK / 4 / NW : (W_TRANS ? BK / 2 / NW : BN * CR / 64 / NW);   // weight side
+    constexpr int WROW = BN * 2;                         // bytes of a [reduction][column] tile row (16-bit)
+    constexpr int QL = W_FP8 ? BK / 4 / NW : (W_TRANS ? BK * WROW / 1024 / NW : BN * CR / 64 / NW);   // weight side
     static_assert(PL >= 1 && QL >= 1 && PL + QL < 16, "loads per slab");
 
-    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? dl_smem_bytes(BM, BK, NSTAGE) : dl_smem_bytes_scatter(BM, BK, NSTAGE)];
+    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? dl_smem_bytes(BM, BN, BK, NSTAGE)
+                                                               : dl_smem_bytes_scatter(BM, BN, BK, NSTAGE)];
     uint32_t *a_voff = reinterpret_cast<uint32_t *>(smem + NSTAGE * STAGE);
     int64_t *c_off = reinterpret_cast<int64_t *>(smem + NSTAGE * STAGE + BM * 4);
 
@@ -140,9 +146,11 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
             const int n = n0 + ((lane & 15) ^ (row & 15)) * 16;
             qv[jj] = n < N ? (uint32_t)row * (uint32_t)N + n : kVoffInvalid;
         } else {
-            // [BK reduction rows][32 chunks]: a load covers 2 rows; lane l lands on row 2j + l/32, physical chunk l%32
-            const int row = (wave * QL + jj) * 2 + (lane >> 5);
-            const int pc = lane & 31;
+            // [BK reduction rows][BN/8 chunks]: a load covers 2 (4) rows of 32 (16) chunks; lane l lands on
+            // row 2j + l/32 (4j + l/16), physical chunk l%32 (l%16)
+            constexpr int LPR = WROW / 16;               // lanes (chunks) per row
+            const int row = (wave * QL + jj) * (64 / LPR) + lane / LPR;
+            const int pc = lane % LPR;
             const int n = n0 + ((((pc >> 1) ^ tr_swizzle(row)) << 1) | (pc & 1)) * 8;
             qv[jj] = n < N ? ((uint32_t)row * (uint32_t)N + n) * 2 : kVoffInvalid;
         }
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
 
     // ---------------- fragment addresses
     const int a = lane & 15, g = lane >> 4;
-    const int wave_m0 = (wave >> 2) * 128, wave_n0 = (wave & 3) * 64;
+    const int wave_m0 = (wave / WN) * 128, wave_n0 = (wave % WN) * 64;
     f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -189,7 +197,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
                 n_at[ks][h] = row * 256 + (((wave_n0 >> 4) ^ (row & 15)) << 4) + (a & 1) * 8;
             } else {
                 const int row = ks * 32 + g * 8 + h * 4 + (a >> 2);
-                n_at[ks][h] = row * 512 + (((wave_n0 >> 4) ^ tr_swizzle(row)) << 5) + (a & 3) * 8;
+                n_at[ks][h] = row * WROW + (((wave_n0 >> 4) ^ tr_swizzle(row)) << 5) + (a & 3) * 8;
             }
         }
 
@@ -274,7 +282,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
         // free now), 128 rows of fp32 (or all 256 rows of a 16-bit type) at a time, and leaves as whole row
         // segments: one store instruction writes 1 KB of one row (fp32) or 512 bytes of each of two rows, which
         // is what the write path wants (product rows are the largest stream of the scatter: 1 GB at C3).
-        // LDS row = 256 columns; its 16-byte chunks are XORed with the low four row bits so that the 16 lanes
+        // LDS row = BN columns; its 16-byte chunks are XORed with the low four row bits so that the 16 lanes
         // of a fragment (16 rows, same chunk) spread over the banks.
         constexpr int ROW_BYTES = BN * OES;                 // 1024 or 512
         constexpr int HALVES = (BM * ROW_BYTES) / (NSTAGE * STAGE) > 1 ? 2 : ((BM * ROW_BYTES > NSTAGE * STAGE) ? 2 : 1);
@@ -285,7 +293,7 @@ __global__ __launch_bounds__(BM * 2) void rows_gemm_dl_kernel(RowsGemmParams p)
     #pragma unroll 1
         for (int half = 0; half < HALVES; ++half) {
             __syncthreads();                                // stages (or the previous pass) no longer being read
-            if (HALVES == 1 || (wave >> 2) == half) {
+            if (HALVES == 1 || (wave / WN) == half) {
                 const int row0 = (HALVES == 1 ? wave_m0 : 0) + a;
     #pragma unroll
                 for (int i = 0; i < TM; ++i) {

@@ -39,14 +39,14 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                             aligned_to(p.C, 16);
             if constexpr (WES == 2 || W_TRANS) {
                 if (dl) {
-                    const size_t smem = GATHER ? 0 : (size_t)dl_smem_bytes_scatter(256, 64, 2);
+                    const size_t smem = GATHER ? 0 : (size_t)dl_smem_bytes_scatter(256, 256, 64, 2);
                     p.csr_threads = 512;            // as many wavefronts as the histograms leave room for
                     while (p.csr_threads > kWave && csr_count_lds(p.T, p.csr_threads / kWave) > smem) p.csr_threads >>= 1;
                     if (GATHER || csr_count_lds(p.T, p.csr_threads / kWave) > smem) p.csr_blocks = 0;
                     grid += p.csr_blocks;
                     if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
                     p.csr_done = p.csr_blocks > 0;
-                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, 256, 64, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(512), 0, s, p);
+                    hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, 256, 256, 64, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(512), 0, s, p);
                     EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
                     return EGS_OK;
                 }
@@ -55,6 +55,23 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                                dim3(512), 0, s, p);
         }
     } else {
+        // 65..191 output columns.  The gathers of large, well-formed 16-bit shapes take the direct-to-LDS
+        // pipeline with 256 x 128 x 64 tiles (four wavefronts, two stages; 32-deep slabs with three workgroups per
+        // CU and a third stage measured the same or slower)
+        if constexpr (TT::ES == 2 && WES == 2 && GATHER && EPI == EPI_STORE) {
+            const bool dl = !g_force_generic && Me >= 512 && p.R >= 128 && p.R % 64 == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
+                            p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && p.w_scale == nullptr && aligned_to(p.C, 16);
+            if (dl) {
+                p.m_tiles = ceil_div(Me, 256); p.n_tiles = ceil_div(p.N, 128);
+                int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
+                if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
+                p.csr_blocks = 0;
+                hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, 2, 256, 128, 64, 2, true, W_TRANS, EPI_STORE>), dim3((unsigned)grid),
+                                   dim3(dl_threads(256, 128)), 0, s, p);
+                EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
+                return EGS_OK;
+            }
+        }
         constexpr int BM = 128, BN = 128;
         p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
         int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;

@@ -33,6 +33,9 @@ SHAPES = [
     (2, 200, 3, 128, 256, 72),    # large weight gradient without splits, 72 of 128 columns
     (3, 100, 5, 200, 256, 128),   # large scatter products with a short reduction (128), ragged last row tile
     (2, 80, 3, 260, 512, 256),    # the same with reduction 256 and two column tiles
+    (3, 100, 5, 200, 128, 256),   # large dY with 128 output columns (256 x 128 tiles, weight stored [column][reduction])
+    (2, 150, 3, 300, 128, 136),   # large gather with 136 output columns: two 128-column tiles, the second nearly empty
+    (2, 150, 3, 300, 136, 128),   # the same for dY
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
