@@ -17,7 +17,7 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
     const int e_groups = ceil_div(p.E, 8);
     // tile shape: 128 x 64 for narrow outputs, 256 x 256 (8 wavefronts) when the product is large
     // enough to be bound by operand traffic (16-bit types), else 128 x 128
-    const bool big = TT::ES == 2 && EPI != EPI_ATOMIC_F32 && p.N >= 192 && Me >= 512 && p.R >= 128;
+    const bool big = TT::ES == 2 && EPI != EPI_ATOMIC_F32 && p.N >= 192 && Me >= 256 && p.R >= 128;
     if (p.N <= 64) {
         constexpr int BM = 128, BN = 64;
         p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
@@ -59,7 +59,7 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
         // pipeline with 256 x 128 x 64 tiles (four wavefronts, two stages; 32-deep slabs with three workgroups per
         // CU and a third stage measured the same or slower)
         if constexpr (TT::ES == 2 && WES == 2 && GATHER && EPI == EPI_STORE) {
-            const bool dl = !g_force_generic && Me >= 512 && p.R >= 128 && p.R % 64 == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
+            const bool dl = !g_force_generic && Me >= 256 && p.R >= 128 && p.R % 64 == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
                             p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && p.w_scale == nullptr && aligned_to(p.C, 16);
             if (dl) {
                 p.m_tiles = ceil_div(Me, 256); p.n_tiles = ceil_div(p.N, 128);

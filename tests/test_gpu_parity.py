@@ -36,6 +36,7 @@ SHAPES = [
     (3, 100, 5, 200, 128, 256),   # large dY with 128 output columns (256 x 128 tiles, weight stored [column][reduction])
     (2, 150, 3, 300, 128, 136),   # large gather with 136 output columns: two 128-column tiles, the second nearly empty
     (2, 150, 3, 300, 136, 128),   # the same for dY
+    (2, 200, 3, 150, 256, 128),   # 300 rows per expert: the smallest products the 256-row tiles are used for
 ]
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
