@@ -40,6 +40,16 @@ inline int elem_size(int dtype)
     }
 }
 
+inline int ind_size(int ind_dtype)
+{
+    switch (ind_dtype) {
+    case EGS_IND_U8: return 1;
+    case EGS_IND_I16: return 2;
+    case EGS_IND_I32: return 4;
+    default: return 8;
+    }
+}
+
 inline int grid_1d(size_t items, int cap = 8192)
 {
     size_t g = (items + kThreads - 1) / kThreads;

@@ -559,6 +559,36 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         if (used) return rc_fused;
     }
 
+    // Product rows that one launch writes and the next reads back are still in the 256 MB memory-side
+    // cache when there are few enough of them.  A call with more is cut into groups of batch elements
+    // (independent of each other) where that leaves every expert at least 1024 rows per group and the
+    // weights, which each group reads again, are small next to the rows (C4: 2 groups, 139 -> 127 us;
+    // smaller groups lose more in the product kernel than the cache gives back).
+    {
+        const bool f32_rows = mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32;
+        const uint64_t per_b = (uint64_t)N * d->I * (f32_rows ? 4 : ES);
+        const uint64_t keep = 144ull << 20;
+        if (per_b > 0 && per_b * d->B > (192ull << 20) && per_b <= keep) {
+            int G = (int)(keep / per_b);
+            const int groups = ceil_div(d->B, G);
+            G = ceil_div(d->B, groups);
+            const uint64_t w_bytes = (uint64_t)d->E * d->I * d->J * ES;
+            if (groups > 1 && (int64_t)G * d->K >= 1024 && w_bytes * (groups - 1) * 4 <= per_b * d->B) {
+                for (int b0 = 0; b0 < d->B; b0 += G) {
+                    egs_dims sub = *d;
+                    sub.B = d->B - b0 < G ? d->B - b0 : G;
+                    const bool last = b0 + G >= d->B;
+                    const int rc = gemm_scatter_impl((const char *)Y + (size_t)b0 * N * d->J * ES,  W,
+                                                     (const char *)Ind + (size_t)b0 * N * ind_size(ind_dtype),
+                                                     (char *)Out + (size_t)b0 * d->T * d->I * ES, workspace, &sub, act_dtype,
+                                                     ind_dtype, w_layout, mode, last ? dw : nullptr, s);
+                    if (rc != EGS_OK) return rc;
+                }
+                return EGS_OK;
+            }
+        }
+    }
+
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
     // gather-and-sum per token that writes every output row exactly once
     int32_t *seg_off = (int32_t *)(ws + pl.seg_off_at);

@@ -119,6 +119,22 @@ def test_c4_zipf_routing_both_modes():
     check_large("C4", ["deterministic", "atomic"])
 
 
+def test_scatter_cut_into_uneven_batch_groups():
+    """20 batch elements of C4's shape: 336 MB of fp32 product rows, which the library processes as
+    groups of 7, 7 and 6 batch elements; elements on both sides of every group boundary against the oracle."""
+    cfg = wl.CONFIGS["C4"]
+    _, T, E, K, I, J = cfg.dims
+    B = 20
+    inp = wl.make_inputs(cfg, dims=(B, T, E, K, I, J))
+    Y = torch.randn(B, E, K, J, generator=torch.Generator().manual_seed(11)).to(cfg.dtype)
+    out = hk.expert_scatter_forward_call(Y.to(DEV), inp["Ws"].to(DEV), inp["Ind"].to(DEV), T, torch.float32)
+    assert torch.equal(out, hk.expert_scatter_forward_call(Y.to(DEV), inp["Ws"].to(DEV), inp["Ind"].to(DEV), T, torch.float32))
+    Indn = inp["Ind"].numpy()
+    for b in (0, 6, 7, 13, 14, 19):
+        ref = O.scatter_forward(np64(Y[b:b + 1]), np64(inp["Ws"]), Indn[b:b + 1], T, acc=np.float64)
+        assert_close(out[b:b + 1], ref, cfg.dtype, f"out[{b}]")
+
+
 def test_c5_fp8_weights_forward():
     cfg = wl.CONFIGS["C5"]
     B, T, E, K, I, J = cfg.dims
