@@ -559,36 +559,6 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         if (used) return rc_fused;
     }
 
-    // Product rows that one launch writes and the next reads back are still in the 256 MB memory-side
-    // cache when there are few enough of them.  A call with more is cut into groups of batch elements
-    // (independent of each other) where that leaves every expert at least 1024 rows per group and the
-    // weights, which each group reads again, are small next to the rows (C4: 2 groups, 139 -> 127 us;
-    // smaller groups lose more in the product kernel than the cache gives back).
-    {
-        const bool f32_rows = mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32;
-        const uint64_t per_b = (uint64_t)N * d->I * (f32_rows ? 4 : ES);
-        const uint64_t keep = 144ull << 20;
-        if (per_b > 0 && per_b * d->B > (192ull << 20) && per_b <= keep) {
-            int G = (int)(keep / per_b);
-            const int groups = ceil_div(d->B, G);
-            G = ceil_div(d->B, groups);
-            const uint64_t w_bytes = (uint64_t)d->E * d->I * d->J * ES;
-            if (groups > 1 && (int64_t)G * d->K >= 1024 && w_bytes * (groups - 1) * 4 <= per_b * d->B) {
-                for (int b0 = 0; b0 < d->B; b0 += G) {
-                    egs_dims sub = *d;
-                    sub.B = d->B - b0 < G ? d->B - b0 : G;
-                    const bool last = b0 + G >= d->B;
-                    const int rc = gemm_scatter_impl((const char *)Y + (size_t)b0 * N * d->J * ES,  W,
-                                                     (const char *)Ind + (size_t)b0 * N * ind_size(ind_dtype),
-                                                     (char *)Out + (size_t)b0 * d->T * d->I * ES, workspace, &sub, act_dtype,
-                                                     ind_dtype, w_layout, mode, last ? dw : nullptr, s);
-                    if (rc != EGS_OK) return rc;
-                }
-                return EGS_OK;
-            }
-        }
-    }
-
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
     // gather-and-sum per token that writes every output row exactly once
     int32_t *seg_off = (int32_t *)(ws + pl.seg_off_at);
@@ -612,13 +582,51 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         rc = launch_rows_small_job(j, dw, s);
     } else {
         rows_f32 = mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32;   // fast mode: rows in the element type
+        // Product rows that one launch writes and the next reads back are still in the 256 MB memory-side
+        // cache when there are few enough of them.  A call with more is processed as groups of batch
+        // elements (independent of each other; the routing tables of all of them are built with the first
+        // group): the largest groups whose rows take at most 144 MB, provided the weights, which every
+        // group reads again, fit beside them and the groups still fill the 256-row tiles of the product
+        // kernel.  C4: 2 groups of 8, 142 -> 123 us; C3: 8 groups of 1, 600 -> 565 us.  Smaller groups than
+        // necessary lose more in the product kernel than the cache returns (C4, groups of 4: 168 us).
+        int G = d->B;
+        {
+            const uint64_t per_b = (uint64_t)N * d->I * (rows_f32 ? 4 : ES);
+            const uint64_t keep = 144ull << 20;
+            if (per_b > 0 && per_b * d->B > (192ull << 20) && per_b <= keep) {
+                const int fit = (int)(keep / per_b);
+                const int groups = ceil_div(d->B, fit);
+                const int g = ceil_div(d->B, groups);
+                const uint64_t w_bytes = (uint64_t)d->E * d->I * d->J * ES;
+                const int64_t rows_e = (int64_t)g * d->K;                     // rows per expert and group
+                const int64_t padded = (rows_e + 255) / 256 * 256;
+                if (groups > 1 && rows_e >= 256 && padded * 100 <= rows_e * 115 && w_bytes <= keep / 2) G = g;
+            }
+        }
         p.C = (char *)rows;
         p.c_vec = d->I % 4 == 0;
-        // the routing table may ride along with the product launch (large shapes); otherwise it is a launch of its own
-        p.csr_blocks = N > 0 ? d->B : 0; p.csr_done = 0;
         p.seg_off = seg_off; p.perm = perm; p.rank_tmp = rank_tmp; p.long_tab = long_tab;
-        rc = rows_gemm_scatter(p, act_dtype, w_trans, rows_f32 ? EPI_STORE_F32 : EPI_STORE, s);
-        if (rc == EGS_OK && !p.csr_done) rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
+        for (int b0 = 0; b0 < d->B; b0 += G) {
+            egs_dims sub = *d;
+            sub.B = d->B - b0 < G ? d->B - b0 : G;
+            p.A = (const char *)Y + (size_t)b0 * N * d->J * ES;
+            p.B = sub.B;
+            const uint64_t span = (uint64_t)sub.B * N * d->J * ES;
+            p.a_bytes = span < (1ull << 31) ? (uint32_t)span : 0;
+            // the routing table may ride along with the (first) product launch (large shapes); otherwise it is a
+            // launch of its own
+            p.csr_blocks = (b0 == 0 && N > 0) ? d->B : 0; p.csr_done = 0;
+            rc = rows_gemm_scatter(p, act_dtype, w_trans, rows_f32 ? EPI_STORE_F32 : EPI_STORE, s);
+            if (rc == EGS_OK && b0 == 0 && !p.csr_done)
+                rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
+            if (rc != EGS_OK) return rc;
+            rc = launch_segment_sum(rows, rows_f32, seg_off + (size_t)b0 * (d->T + 1), perm + (size_t)b0 * N,
+                                    long_tab + (size_t)b0 * long_tab_stride(N), long_part + (size_t)b0 * long_max_slots(N) * d->I,
+                                    (char *)Out + (size_t)b0 * d->T * d->I * ES, &sub, act_dtype,
+                                    b0 + G >= d->B ? dw : nullptr, s);
+            if (rc != EGS_OK) return rc;
+        }
+        return EGS_OK;
     }
     if (rc != EGS_OK) return rc;
     return launch_segment_sum(rows, rows_f32, seg_off, perm, long_tab, long_part, Out, d, act_dtype, dw, s);
