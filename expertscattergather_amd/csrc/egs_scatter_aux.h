@@ -553,15 +553,30 @@ __device__ __forceinline__ void segment_sum_long_body(const SegSumParams &sp, co
         float acc[VW];
 #pragma unroll
         for (int x = 0; x < VW; ++x) acc[x] = 0.f;
-        for (int cc = 0; cc < nch; ++cc) {
-            const float *src = pt + (size_t)cc * I + (size_t)iv * VW;
+        // eight partial rows in flight at a time; added in chunk order all the same
+        for (int c0 = 0; c0 < nch; c0 += 8) {
             if constexpr (VW == 4) {
-                const uint64_t lo = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                const uint64_t hi = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                acc[0] += bits_f32((uint32_t)lo); acc[1] += bits_f32((uint32_t)(lo >> 32));
-                acc[2] += bits_f32((uint32_t)hi); acc[3] += bits_f32((uint32_t)(hi >> 32));
+                uint64_t lo[8], hi[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const float *src = pt + (size_t)min(c0 + u, nch - 1) * I + (size_t)iv * VW;
+                    lo[u] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    hi[u] = __hip_atomic_load(reinterpret_cast<const uint64_t *>(src) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (c0 + u < nch) {
+                        acc[0] += bits_f32((uint32_t)lo[u]); acc[1] += bits_f32((uint32_t)(lo[u] >> 32));
+                        acc[2] += bits_f32((uint32_t)hi[u]); acc[3] += bits_f32((uint32_t)(hi[u] >> 32));
+                    }
             } else {
-                acc[0] += __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                float v[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    v[u] = __hip_atomic_load(pt + (size_t)min(c0 + u, nch - 1) * I + iv, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (c0 + u < nch) acc[0] += v[u];
             }
         }
         const size_t at = ((size_t)b * T + t) * I + (size_t)iv * VW;
