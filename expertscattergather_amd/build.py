@@ -20,6 +20,9 @@ HIPCC_FLAGS = [
     "-munsafe-fp-atomics",                      # fp32 atomic add as one hardware instruction
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",   # no packed-fp32 VALU ops
     "-Wall", "-Wno-unused-function",
+    # the direct-to-LDS loads are inline assembly that sets M0 (the LDS base of the load) and names it as
+    # clobbered; the compiler warns once per instantiation that M0 is a reserved register
+    "-Wno-inline-asm",
 ]
 NOISE = "is not a recognized feature for this target"
 
