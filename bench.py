@@ -31,7 +31,10 @@ MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
 # runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
 # Counters cannot be read from inside this process, so the figure is the recorded one.
 MEASURED_TRAFFIC_BYTES = {("C2", "gather_gemm"): 17349000,        # profiles/rows_small_gather_c2_traffic.md
-                          ("C3", "gather_gemm"): 693100000}       # profiles/rows_gemm_dl_gather_c3_counters.md
+                          ("C3", "gather_gemm"): 693100000,       # profiles/rows_gemm_dl_gather_c3_counters.md
+                          ("C1", "gather_gemm"): 46310000,        # profiles/gather_traffic_c1_c4_c5.md
+                          ("C4", "gather_gemm"): 80920000,
+                          ("C5", "gather_gemm"): 2922340000}
 
 
 def parse_args():
@@ -77,8 +80,13 @@ def main():
         dst = torch.empty_like(src)
         for _ in range(3):
             dst.copy_(src)
+        if args.config == "C5":     # the configuration's own weights: e4m3 bytes and fp32 scales
+            Wq_p, scale_p = (t.to(dev) for t in wl.quantize_fp8_weights(inp["Wg"].float()))
         for _ in range(5):
-            hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+            if args.config == "C5":
+                hk.expert_gather_fp8w_forward(X, Wq_p, scale_p, Ind)
+            else:
+                hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
         torch.cuda.synchronize()
         print(json.dumps({"pmc_probe": True, "copy_bytes_read": 64 << 20, "copy_bytes_written": 64 << 20}))
         return
