@@ -8,7 +8,9 @@
 //     right after the barrier that publishes slab k and land while the MFMAs run.  One barrier
 //     per slab.  The shape in use is 256 x 256 x 64 with two stages (one 134 KB workgroup per CU, fewest
 //     bytes moved per flop); 128 x 256 x 32 with two or three stages (two or three workgroups per
-//     CU) compiles as well but measured slower on every benchmark configuration.
+//     CU) and 256 x 256 x 32 with four stages compile as well but measured slower on every benchmark
+//     configuration (the loads are bound by bandwidth beyond the L2, not by latency, and 32-deep slabs
+//     pay twice the barriers).
 //   * Rows that are fetched through Ind are just per-lane byte offsets into the buffer
 //     descriptor; rows that do not exist get an offset outside it and arrive as zeros.
 //   * K-major operands ([row][reduction]) are read back with 16-byte LDS reads (XOR swizzle set
@@ -57,7 +59,7 @@ __global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGe
     static_assert(EPI == EPI_STORE || EPI == EPI_STORE_F32, "plain stores only");
     static_assert(WES == 2 || (WES == 1 && W_TRANS && TT::ID == 2), "fp8 weights: [reduction][column] layout, widened to bf16");
     static_assert((BM == 128 || BM == 256) && (BN == 128 || BN == 256) && (BK == 32 || BK == 64) &&
-                  (NSTAGE == 2 || NSTAGE == 3), "tile shapes");
+                  (NSTAGE >= 2 && NSTAGE <= 4), "tile shapes");
     constexpr bool W_FP8 = (WES == 1);
     static_assert(!W_FP8 || BN == 256, "the fp8 tile layout is written for 256-byte rows");
     constexpr int WN = BN / 64;                          // wavefront columns
@@ -208,8 +210,12 @@ __global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGe
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt) {
         // slab kt has landed once at most the loads of the slabs issued after it are outstanding
-        if (NSTAGE == 3 && kt + 1 < nk) wait_vmem<(NSTAGE == 3 ? PL + QL : 0)>();
-        else wait_vmem<0>();
+        {
+            const int later = min(nk - 1 - kt, NSTAGE - 2);     // slabs requested after slab kt that may stay in flight
+            if (NSTAGE >= 4 && later >= 2) wait_vmem<(NSTAGE >= 4 ? 2 * (PL + QL) : 0)>();
+            else if (NSTAGE >= 3 && later >= 1) wait_vmem<(NSTAGE >= 3 ? PL + QL : 0)>();
+            else wait_vmem<0>();
+        }
         __syncthreads();            // slab kt visible to all; everyone is done reading the stage refilled next
         if (kt + NSTAGE - 1 < nk) {
             int fill = stage + NSTAGE - 1;
@@ -218,29 +224,58 @@ __global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGe
         }
         const char *tile_m = smem + stage * STAGE;
         const char *tile_n = tile_m + P_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < KSTEPS; ++ks) {
-            u32x4 mf[TM], nf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) mf[i] = *reinterpret_cast<const u32x4 *>(tile_m + m_at[ks] + i * (16 * BK * 2));
+        // Fragment reads run one step ahead of the MFMAs that use them: the row fragments of the next pair
+        // of 16-row tiles (and, at the end of a reduction step, the weight fragments of the next step) are
+        // requested before the eight MFMAs of the current pair are issued, so a wavefront's LDS latency is
+        // covered by its own MFMAs instead of stalling them.
+        auto read_n = [&](int ks, u32x4 (&nr)[TN]) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 if constexpr (!W_TRANS) {
-                    nf[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][0] + j * (16 * BK * 2));
+                    nr[j] = *reinterpret_cast<const u32x4 *>(tile_n + n_at[ks][0] + j * (16 * BK * 2));
                 } else if constexpr (W_FP8) {
-                    u32x2 q8 = lds_read_tr8(tile_n + (n_at[ks][0] ^ (j << 4)));      // chunk wave_n0/16 + j, j < 4
-                    nf[j] = fp8x8_to_bf16_chunk(q8[0], q8[1]);
+                    const u32x2 q8 = lds_read_tr8(tile_n + (n_at[ks][0] ^ (j << 4)));       // chunk wave_n0/16 + j, j < 4
+                    nr[j] = u32x4{q8[0], q8[1], 0u, 0u};                                    // widened at first use
                 } else {
                     // unit wave_n0/16 + j: wave_n0/16 is a multiple of 4 and j < 4, so j folds in by XOR
-                    u32x2 lo = lds_read_tr16(tile_n + (n_at[ks][0] ^ (j << 5)));
-                    u32x2 hi = lds_read_tr16(tile_n + (n_at[ks][1] ^ (j << 5)));
-                    nf[j] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+                    const u32x2 lo = lds_read_tr16(tile_n + (n_at[ks][0] ^ (j << 5)));
+                    const u32x2 hi = lds_read_tr16(tile_n + (n_at[ks][1] ^ (j << 5)));
+                    nr[j] = u32x4{lo[0], lo[1], hi[0], hi[1]};
                 }
             }
+        };
+        auto read_m2 = [&](int ks, int ip, u32x4 (&mr)[2]) {
+            mr[0] = *reinterpret_cast<const u32x4 *>(tile_m + m_at[ks] + (2 * ip) * (16 * BK * 2));
+            mr[1] = *reinterpret_cast<const u32x4 *>(tile_m + m_at[ks] + (2 * ip + 1) * (16 * BK * 2));
+        };
+        constexpr int PAIRS = TM / 2;
+        u32x4 nraw[2][TN], mf[2][2];
+        read_n(0, nraw[0]);
+        read_m2(0, 0, mf[0]);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            u32x4 nf[TN];
 #pragma unroll
-                for (int j = 0; j < TN; ++j) mma_chunk<TT>(acc[i][j], nf[j], mf[i]);
+            for (int j = 0; j < TN; ++j) {
+                if constexpr (W_FP8) nf[j] = fp8x8_to_bf16_chunk(nraw[ks & 1][j][0], nraw[ks & 1][j][1]);
+                else nf[j] = nraw[ks & 1][j];
+            }
+#pragma unroll
+            for (int ip = 0; ip < PAIRS; ++ip) {
+                const int cur = (ks * PAIRS + ip) & 1;
+                if (ip + 1 < PAIRS) {
+                    read_m2(ks, ip + 1, mf[cur ^ 1]);
+                } else if (ks + 1 < KSTEPS) {
+                    read_n(ks + 1, nraw[(ks + 1) & 1]);
+                    read_m2(ks + 1, 0, mf[cur ^ 1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);      // the requests above stay ahead of the MFMAs below
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) mma_chunk<TT>(acc[2 * ip + h][j], nf[j], mf[cur][h]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
         if (++stage == NSTAGE) stage = 0;
     }
