@@ -118,3 +118,15 @@ def test_expert_choice_router_picks_top_k_tokens_per_expert():
         expert_choice_router(torch.randn(1, 300, 2), 2, torch.uint8)      # ids up to 299 do not fit
     with pytest.raises(ValueError):
         expert_choice_router(logits, T + 1)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """`bench.py --gpus N` with N above 1 exits with a message instead of measuring anything."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                         timeout=120)
+    assert res.returncode != 0
+    assert "one GPU" in res.stderr and res.stdout.strip() == ""
