@@ -112,7 +112,7 @@ def check_large(name, modes):
 
 
 def test_c3_long_sequence_bf16():
-    check_large("C3", ["deterministic"])
+    check_large("C3", ["deterministic", "atomic"])
 
 
 def test_c4_zipf_routing_both_modes():
