@@ -168,8 +168,10 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int q = q_begin + c * kWave + lane;
-        const int32_t t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);     // unconditional: loads overlap
-        tk[c] = (in_regs && q < q_end) ? t : -1;
+        int32_t t = -1;
+        if (in_regs && c * kWave < slice)        // uniform; within the slice the loads are unconditional so that they overlap
+            t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);
+        tk[c] = q < q_end ? t : -1;
         rk[c] = 0;
     }
     after_token_loads();        // whatever else the caller wants in flight while the tokens travel

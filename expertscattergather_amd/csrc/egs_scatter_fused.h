@@ -79,7 +79,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     Unit buf[kFusedDepth];
     const uint32_t a_base_b = (uint32_t)b * (uint32_t)NP * R * ES;
     auto load_unit = [&](Unit &u, int unit) {
-        unit = min(unit, units - 1);                    // unconditional loads; surplus units are not stored
+        if (unit >= units) return;                      // uniform per wavefront; a unit's own loads are unconditional
         const int e = unit / KT2, rp = unit - e * KT2;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
