@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 # MI355X dense matrix peaks (TFLOP/s) of the arithmetic each configuration multiplies in
-MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0}
 
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
@@ -44,6 +44,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="C2", help="workload (C2 = the metric's configuration)")
     ap.add_argument("--mode", default=None, choices=["deterministic", "atomic"], help="scatter mode (default: env / deterministic)")
+    ap.add_argument("--fp8-act", action="store_true",
+                    help="C5 only: quantise the activations per row to e4m3 and multiply on the fp8 matrix instruction")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
@@ -92,12 +94,18 @@ def main():
         return
 
     fp8 = args.config == "C5"
+    if args.fp8_act and not fp8:
+        print("bench.py: --fp8-act applies to the fp8-weight configuration C5 only", file=sys.stderr)
+        sys.exit(2)
+    fp8_act = fp8 and args.fp8_act
     if fp8:     # the configuration's weights: e4m3 bytes and a per-expert, per-column fp32 scale
         Wq_c, scale_c = wl.quantize_fp8_weights(inp["Wg"].float())
         Wq, Wscale = Wq_c.to(dev), scale_c.to(dev)
 
     def step():
-        if fp8:
+        if fp8_act:
+            Y = hk.expert_gather_fp8_forward(X, Wq, Wscale, Ind)
+        elif fp8:
             Y = hk.expert_gather_fp8w_forward(X, Wq, Wscale, Ind)
         else:
             Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
@@ -158,7 +166,13 @@ def main():
     mode = 0 if hk.get_scatter_mode() == "deterministic" else 1
     ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    f8ws_bytes = lib.egs_gather_gemm_fp8act_workspace_bytes(d) if fp8_act else 0
+    f8ws = torch.empty(max(f8ws_bytes, 256), dtype=torch.uint8, device=dev)
+
     def k_gather():
+        if fp8_act:     # row quantiser + fp8 x fp8 product: both launches are part of the call
+            return lib.egs_gather_gemm_fp8act(X.data_ptr(), Wq.data_ptr(), Wscale.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
+                                              f8ws.data_ptr(), f8ws_bytes, d, T * I, I, 2, stream)
         if fp8:
             return lib.egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), Wscale.data_ptr(), d, T * I, I, dt, 3, 2, 0, stream)
         return lib.egs_gather_gemm(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), None, d, T * I, I, dt, dt, 2, 0, stream)
@@ -220,7 +234,7 @@ def main():
     kflops = wl.flops(dims)
     chain_flops = n_equiv * kflops
     dtype_name = "bf16" if cfg.dtype == torch.bfloat16 else ("f16" if cfg.dtype == torch.float16 else "f32")
-    mfma_peak = MFMA_PEAK_TFLOPS[dtype_name]
+    mfma_peak = MFMA_PEAK_TFLOPS["fp8" if fp8_act else dtype_name]
     # the roof that binds a kernel is the slower of "move the algorithmic bytes at 8 TB/s" and
     # "do the flops at the dense matrix peak of the arithmetic type"
     t_hbm, t_mfma = dom_bytes / (HBM_PEAK_GBPS * 1e9), kflops / (mfma_peak * 1e12)
@@ -271,7 +285,8 @@ def main():
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": dtype_name + (" (fp8 e4m3 weights)" if fp8 else ""),
+        "dtype": ("fp8 (e4m3 weights, activations quantised per row to e4m3, fp32 accumulation)" if fp8_act
+                  else dtype_name + (" (fp8 e4m3 weights)" if fp8 else "")),
         "data": "synthetic",
         "config": {"workload": f"{cfg.name}: B{B} T{T} E{E} K{K} I{I} J{J} {cfg.what}", "scatter_mode": hk.get_scatter_mode(),
                    "launch": "hip graph replay" if use_graph else "eager launches through the Python ops"},
@@ -293,7 +308,7 @@ def main():
                      if bound == "hbm" else
                      {"bound": "mfma", "kernel": dom, "achieved": round(kflops / dom_s * 1e-12, 2), "peak": mfma_peak,
                       "unit": "TFLOP/s", "frac": round(kflops / dom_s * 1e-12 / mfma_peak, 4),
-                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
+                      "traffic": None if fp8_act else MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
                       "algorithmic_flops": kflops, "avg_launch_us": round(dom_s * 1e6, 3)}),
         "cpu_baseline": cpu,
     }

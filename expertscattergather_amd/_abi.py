@@ -42,6 +42,8 @@ SIGNATURES = {
     "egs_gather_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "egs_gemm_scatter": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _i, _vp]),
     "egs_dw": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
+    "egs_gather_gemm_fp8act_workspace_bytes": (_sz, [_dp]),
+    "egs_gather_gemm_fp8act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _vp]),
     "egs_expert_gather_forward": (_i, [_vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _vp]),
     "egs_expert_gather_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _i, _vp]),
     "egs_expert_scatter_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _vp]),

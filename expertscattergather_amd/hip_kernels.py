@@ -25,7 +25,7 @@ from . import _abi
 
 __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
-    "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "validate_indices",
+    "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
 ]
 
 OP_NAMESPACE = "egs_amd"
@@ -369,6 +369,43 @@ def expert_gather_fp8w_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.T
                                         _stream_ptr(dev))
     _abi.check(rc, "expert_gather_fp8w_forward")
     return Y
+
+
+def expert_gather_fp8_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.Tensor, Ind: torch.Tensor,
+                              return_quantised: bool = False):
+    """Inference-only gather with fp8 weights and fp8 activations on the fp8 matrix instruction.
+
+    Every row X[b,t,:] is quantised once to float8_e4m3fn with its own scale xs[b,t] = max|X[b,t,:]| / 448, then
+    Y[b,e,k,:] = xs[b,t] * scale[e,:] * (Xq[b,t,:] . Wq[e]) with fp32 accumulation, t = Ind[b,e,k].
+    X is bfloat16 [B,T,I] (I a multiple of 128); Wq is float8_e4m3fn [E,I,J] (J a multiple of 16); scale is
+    float32 [E,J].  With ``return_quantised`` the quantised rows [B,T,I] and their scales [B,T] are returned too."""
+    dev = _require_gpu(X, Wq, scale, Ind)
+    if X.dtype != torch.bfloat16 or Wq.dtype != torch.float8_e4m3fn or scale.dtype != torch.float32:
+        raise ValueError("fp8 gather needs bfloat16 X, float8_e4m3fn W and float32 scale")
+    B, E, K, I, J = _check_shapes(X, Wq, Ind, None, True)
+    if tuple(scale.shape) != (E, J):
+        raise ValueError(f"scale must be [E={E},J={J}], got {tuple(scale.shape)}")
+    X, ld_b, ld_t = _rows_source(X)
+    T = X.shape[1]
+    Wq = Wq.contiguous(); scale = scale.contiguous(); Ind = Ind.contiguous()
+    Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
+    d = _abi.Dims(B, T, E, K, I, J)
+    nbytes = _abi.lib().egs_gather_gemm_fp8act_workspace_bytes(d)
+    if return_quantised:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        ws_ptr = ws.data_ptr()
+    else:
+        ws, (ws_ptr, _) = None, _workspace(dev, nbytes)
+    with _on_device(dev):
+        rc = _abi.lib().egs_gather_gemm_fp8act(X.data_ptr(), Wq.data_ptr(), scale.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
+                                               ws_ptr, nbytes, d, ld_b, ld_t, _ind_type_id(Ind), _stream_ptr(dev))
+    _abi.check(rc, "expert_gather_fp8_forward")
+    if not return_quantised:
+        return Y
+    xq_bytes = (B * T * I + 255) // 256 * 256
+    Xq = ws[:B * T * I].view(torch.float8_e4m3fn).view(B, T, I)
+    xs = ws[xq_bytes:xq_bytes + B * T * 4].view(torch.float32).view(B, T)
+    return Y, Xq, xs
 
 
 def validate_indices(Ind: torch.Tensor, T: int) -> int:

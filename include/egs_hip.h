@@ -138,6 +138,23 @@ int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
            int64_t ldx_b, int64_t ldx_t,
            int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream);
 
+/* Inference variant of the gather with fp8 weights AND fp8 activations, on the fp8 matrix instruction:
+ *   Y[b,e,k,j] = xs[b,t] * w_scale[e,j] * sum_i Xq[b,t,i] * Wq(e,i,j),   t = Ind[b,e,k],
+ * where every source row X[b,t,:] is first quantised to e4m3 (round to nearest even) with its own scale
+ * xs[b,t] = max|X[b,t,:]| / 448 (1 for an all-zero row).  Both steps run on `stream`; the quantised rows and
+ * their scales live in the workspace (egs_gather_gemm_fp8act_workspace_bytes(), 256-byte aligned).
+ * No counterpart in the reference, whose expert_gather_kernel (egs/triton_kernels.py:49-143) takes
+ * fp32/fp16/bf16 only (:15-23); a different numerical contract from egs_gather_gemm with fp8 weights, which
+ * keeps the activations in bf16.
+ *   X    [B,T,I] bf16, strides (ldx_b, ldx_t, 1) in elements, multiples of 8;  I % 128 == 0
+ *   Wq   [E,I,J] e4m3fn;  w_scale float [E,J];  J % 16 == 0
+ *   Y    [B,E,K,J] bf16, dense
+ * Shapes outside these limits return EGS_ERR_UNSUPPORTED. */
+size_t egs_gather_gemm_fp8act_workspace_bytes(const egs_dims *d);
+int egs_gather_gemm_fp8act(const void *X, const void *Wq, const float *w_scale, const void *Ind, void *Y,
+                           void *workspace, size_t workspace_bytes, const egs_dims *d,
+                           int64_t ldx_b, int64_t ldx_t, int ind_dtype, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Launcher-level entry points (one per reference callable)
  * ------------------------------------------------------------------------------------- */

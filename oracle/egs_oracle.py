@@ -34,6 +34,11 @@ fp8 weights (not in the reference; defined by the benchmark configuration that s
 e4m3 with one fp32 scale per expert and output column): the oracle dequantises
 ``W[e,i,j] = fp8_to_float(Wq[e,i,j]) * scale[e,j]`` and runs the ordinary gather.  The
 decode table is checked against ``torch.float8_e4m3fn`` in the tests.
+
+fp8 activations (not in the reference either): every source row is quantised to e4m3 with its
+own scale ``max|row| / 448`` (``quantize_rows_e4m3``: float32 arithmetic, round to nearest even
+by search over the 256-entry decode table, checked against ``torch.float8_e4m3fn``), then the
+oracle dequantises rows and weights and runs the ordinary gather (``gather_forward_fp8``).
 """
 from __future__ import annotations
 
@@ -43,7 +48,8 @@ __all__ = [
     "gather_forward", "scatter_forward", "gather_backward", "scatter_backward",
     "brute_gather_forward", "brute_scatter_forward", "brute_gather_backward",
     "brute_scatter_backward", "fp8_e4m3fn_to_float", "dequant_fp8_weights",
-    "gather_forward_fp8w", "round_to_bf16", "round_to_f16",
+    "gather_forward_fp8w", "float_to_fp8_e4m3fn", "quantize_rows_e4m3", "gather_forward_fp8",
+    "round_to_bf16", "round_to_f16",
 ]
 
 
@@ -253,3 +259,41 @@ def dequant_fp8_weights(Wq_bits, scale) -> np.ndarray:
 def gather_forward_fp8w(X, Wq_bits, scale, Ind, acc=np.float64):
     """Dequantise-then-einsum reference for the fp8-weight gather."""
     return gather_forward(X, dequant_fp8_weights(Wq_bits, scale), Ind, acc=acc)
+
+
+# ----------------------------------------------------------------------------- fp8 activations
+def float_to_fp8_e4m3fn(x) -> np.ndarray:
+    """Encode finite values of magnitude <= 448 as OCP e4m3fn bytes, round to nearest, ties to even.
+
+    Works on the decode table: the two neighbouring codes of |x| are found by search, the nearer one
+    wins and a tie goes to the code with an even mantissa (even byte value: consecutive codes
+    alternate parity)."""
+    x = np.asarray(x, dtype=np.float64)
+    mags = fp8_e4m3fn_to_float(np.arange(0x7F, dtype=np.uint8))        # codes 0x00..0x7e, increasing, 0x7e = 448
+    a = np.abs(x)
+    if a.size and a.max() > 448.0:
+        raise ValueError("magnitude above the e4m3 maximum")
+    hi = np.clip(np.searchsorted(mags, a, side="left"), 0, 0x7E)      # first code >= |x|
+    lo = np.maximum(hi - 1, 0)
+    d_hi, d_lo = mags[hi] - a, a - mags[lo]
+    pick_lo = (d_lo < d_hi) | ((d_lo == d_hi) & (lo % 2 == 0))
+    code = np.where(pick_lo, lo, hi).astype(np.uint8)
+    return np.where(np.signbit(x), code | 0x80, code).astype(np.uint8)
+
+
+def quantize_rows_e4m3(X):
+    """Per-row e4m3 quantisation of X[..., I] in float32 arithmetic: scale = max|row| / 448 (1 for a zero
+    row), q = encode(clamp(x * (1 / scale), -448, 448)).  Returns (bytes [..., I], scale [...])."""
+    X = np.asarray(X, dtype=np.float32)
+    amax = np.abs(X).max(axis=-1)
+    scale = np.where(amax > 0, amax / np.float32(448.0), np.float32(1.0)).astype(np.float32)
+    inv = (np.float32(1.0) / scale).astype(np.float32)
+    y = np.clip((X * inv[..., None]).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    return float_to_fp8_e4m3fn(y), scale
+
+
+def gather_forward_fp8(X, Wq_bits, scale, Ind, acc=np.float64):
+    """fp8-activation, fp8-weight gather: rows quantised per row, both sides dequantised exactly, ordinary gather."""
+    q, xs = quantize_rows_e4m3(X)
+    Xd = fp8_e4m3fn_to_float(q) * xs[..., None].astype(np.float64)
+    return gather_forward(Xd, dequant_fp8_weights(Wq_bits, scale), Ind, acc=acc)

@@ -392,6 +392,46 @@ def test_fp8_weight_gather_matches_dequantised_oracle():
     assert_close(Y, ref, torch.bfloat16, "fp8 weights large")
 
 
+@pytest.mark.parametrize("shape,ind_dtype,oob", [((2, 40, 3, 50, 128, 64), torch.int64, False),
+                                                  ((3, 300, 9, 100, 256, 272), torch.int32, True),
+                                                  ((2, 64, 8, 256, 384, 512), torch.int16, False)],
+                         ids=["one-slab", "ragged-tiles", "full-tiles"])
+def test_fp8_activation_gather_matches_quantised_oracle(shape, ind_dtype, oob):
+    """fp8 x fp8 gather: the row quantiser is bit-exact against the oracle's, the product matches the oracle
+    on the quantised operands to bf16 output accuracy, and stays within 5e-2 relative RMS (the stated bound of
+    per-row e4m3 activations) of the fp8-weight gather that keeps bf16 activations."""
+    from expertscattergather_amd import workloads as wl
+    B, T, E, K, I, J = shape
+    case = make_case(41, B, T, E, K, I, J, torch.bfloat16, ind_dtype=ind_dtype)
+    case["X"][0, 0] = 0                                      # an all-zero row: scale 1
+    if oob:
+        case["Ind"][0, 0, 0] = T + 3                         # contributes a zero row
+        case["Ind"][1, 2, 5] = -1
+    Wq, scale = wl.quantize_fp8_weights(case["Wg"].float())
+    Y, Xq, xs = hk.expert_gather_fp8_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]), return_quantised=True)
+    q_o, xs_o = O.quantize_rows_e4m3(case["X"].float().numpy())
+    assert np.array_equal(xs.cpu().numpy(), xs_o)
+    assert np.array_equal(Xq.cpu().view(torch.uint8).numpy(), q_o)
+    bits = Wq.view(torch.uint8).numpy()
+    ind = case["Ind"].numpy().astype(np.int64)
+    live = (ind >= 0) & (ind < T)
+    safe = np.where(live, ind, 0)
+    ref = O.gather_forward_fp8(case["X"].float().numpy(), bits, scale.numpy(), safe) * live[..., None]
+    assert_close(Y, ref, torch.bfloat16, "fp8 activations")
+    assert torch.equal(Y, hk.expert_gather_fp8_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"])))
+    ref_bf16_act = O.gather_forward_fp8w(np64(case["X"]), bits, scale.numpy(), safe) * live[..., None]
+    rel_rms = np.sqrt(((np64(Y) - ref_bf16_act) ** 2).mean() / (ref_bf16_act ** 2).mean())
+    assert rel_rms <= 5e-2, rel_rms
+
+
+def test_fp8_activation_gather_rejects_shapes_outside_its_tile_layout():
+    from expertscattergather_amd import workloads as wl
+    case = make_case(43, 2, 16, 2, 4, 96, 32, torch.bfloat16)   # I not a multiple of 128
+    Wq, scale = wl.quantize_fp8_weights(case["Wg"].float())
+    with pytest.raises(RuntimeError, match="unsupported"):
+        hk.expert_gather_fp8_forward(dev(case["X"]), dev(Wq), dev(scale), dev(case["Ind"]))
+
+
 def test_ops_pass_opcheck_and_router_output_feeds_the_kernels():
     # registration of the four ops (schema, fake implementations, no hidden mutation), the counterpart of the
     # reference's ~220 lines of torch.library glue (egs/triton_kernels.py:361-578)

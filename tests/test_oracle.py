@@ -170,3 +170,31 @@ def test_fp8_decode_table_matches_torch():
 def test_bf16_rounding_matches_torch():
     a = np.random.default_rng(0).standard_normal(4096).astype(np.float32) * 37
     np.testing.assert_array_equal(O.round_to_bf16(a), torch.from_numpy(a).to(torch.bfloat16).to(torch.float32).numpy())
+
+
+def test_fp8_encoder_and_row_quantiser_match_torch():
+    """Pins float_to_fp8_e4m3fn / quantize_rows_e4m3 against torch's float8_e4m3fn cast (round to nearest even),
+    including every code, every midpoint between codes, subnormals and the zero row."""
+    codes = torch.arange(256, dtype=torch.uint8)
+    vals = codes.view(torch.float8_e4m3fn).float()
+    finite = ~torch.isnan(vals)
+    assert np.array_equal(O.float_to_fp8_e4m3fn(vals[finite].numpy())[vals[finite] != 0], codes[finite][vals[finite] != 0].numpy())
+    mags = vals[:0x7F]
+    mids = (mags[:-1] + mags[1:]) / 2                        # exact in float32: ties
+    g = torch.Generator().manual_seed(5)
+    x = torch.cat([mids, -mids, torch.rand(20000, generator=g) * 896 - 448, torch.randn(20000, generator=g) * 0.02,
+                   torch.tensor([0.0, -0.0, 448.0, -448.0, 2.0 ** -9, 2.0 ** -10, 3 * 2.0 ** -11])])
+    ours = O.float_to_fp8_e4m3fn(x.numpy())
+    theirs = x.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(ours, theirs)
+    X = torch.randn(7, 5, 64, generator=g).to(torch.bfloat16)
+    X[2, 3] = 0
+    X[1, 1] *= 1e-3
+    q, xs = O.quantize_rows_e4m3(X.float().numpy())
+    amax = X.float().abs().amax(dim=-1)
+    xs_t = torch.where(amax > 0, amax / 448.0, torch.ones_like(amax))
+    q_t = (X.float() * (1.0 / xs_t)[..., None]).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    assert np.array_equal(xs, xs_t.numpy()) and np.array_equal(q, q_t.numpy())
+    # a quantised row reproduces the row to e4m3 accuracy: |x - dequant| <= 2^-4 |x| + half a subnormal step
+    deq = O.fp8_e4m3fn_to_float(q) * xs[..., None]
+    assert (np.abs(deq - X.float().numpy()) <= 2.0 ** -4 * np.abs(X.float().numpy()) + xs[..., None] * 2.0 ** -10).all()
