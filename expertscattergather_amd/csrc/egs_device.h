@@ -108,16 +108,29 @@ template <> __device__ __forceinline__ void mma_chunk<ElemF32>(f32x4 &acc, const
 // several index loads can be in flight): one 8-byte load of the aligned window that contains the
 // element, then shift and sign- or zero-extend.  The window never leaves the allocation because
 // device allocations start and end on multiples of 8 bytes and elements are naturally aligned.
-__device__ __forceinline__ int64_t load_index_raw(const void *ind, int ind_dtype, int64_t at)
+// The load and the decoding are separate functions so that a kernel can put other loads between them.
+__device__ __forceinline__ uint64_t load_index_word(const void *ind, int ind_dtype, int64_t at)
 {
     const int es_log2 = (0x0321 >> (4 * ind_dtype)) & 0xF;          // int16 -> 1, int32 -> 2, int64 -> 3, uint8 -> 0
+    // pointer arithmetic on `ind` itself (not on its integer value): the compiler then knows the load is a
+    // global one, which returns in order with the other global loads of the wavefront
+    const int64_t mis = (int64_t)(reinterpret_cast<uint64_t>(ind) & 7ull);
+    const int64_t off = (at << es_log2) + mis;
+    return *reinterpret_cast<const uint64_t *>(static_cast<const char *>(ind) - mis + (off & ~(int64_t)7));
+}
+__device__ __forceinline__ int64_t decode_index_word(uint64_t w, const void *ind, int ind_dtype, int64_t at)
+{
+    const int es_log2 = (0x0321 >> (4 * ind_dtype)) & 0xF;
     const uint64_t addr = reinterpret_cast<uint64_t>(ind) + ((uint64_t)at << es_log2);
-    uint64_t w = *reinterpret_cast<const uint64_t *>(addr & ~7ull);
     const int bits = 8 << es_log2;
     w <<= 64 - bits - (int)(addr & 7ull) * 8;                       // element now in the top `bits` bits
     const int64_t sx = (int64_t)w >> (64 - bits);                   // sign-extended
     const int64_t zx = (int64_t)(w >> (64 - bits));                 // zero-extended (uint8)
     return ind_dtype == 3 ? zx : sx;
+}
+__device__ __forceinline__ int64_t load_index_raw(const void *ind, int ind_dtype, int64_t at)
+{
+    return decode_index_word(load_index_word(ind, ind_dtype, at), ind, ind_dtype, at);
 }
 __device__ __forceinline__ int32_t load_token(const void *ind, int ind_dtype, int64_t at, int32_t T)
 {

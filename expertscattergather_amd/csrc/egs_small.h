@@ -72,6 +72,17 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     const int N = p.N;
     if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)block * 4 + wave) * 2] = wall_clock64();
 
+    // Order of the loads.  Loads return in order, and the long chain is index -> row.  So the index load goes
+    // first, the weight loads follow in the shadow of its latency, and the row loads are issued as soon as the
+    // index is there (the wait names the index load alone); the weight blocks are transposed only after that.
+    // this lane's pick (row m0 + lane): byte offsets of its source row and of its result row
+    const int m_lane = m0 + lane;
+    const int mm_lane = min(m_lane, Me - 1);
+    const int b_lane = mm_lane / p.K;
+    const int64_t pick = ((int64_t)b_lane * p.E + e) * p.K + (mm_lane - b_lane * p.K);
+    uint64_t t_word = 0;
+    if constexpr (GATHER) t_word = load_index_word(p.Ind, p.ind_dtype, pick);
+
     // Which output column does accumulator row a' = 4g+r of MFMA tile tn hold?  Chosen so that
     // in every store instruction the four lanes g = 0..3 of one result row write one contiguous
     // 64-byte run (16 bytes each); the weight fragments are loaded to match.
@@ -82,36 +93,29 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     //       16-bit, TN == 4     one 4-col block:  starts at 32*((a'/2)%2) + 8*(a'/4) + 4*(a'%2)
     //       16-bit, TN == 8     one 8-col block:  starts at 32*(a'%4) + 8*(a'/4)
     const char *We = p.W + (size_t)e * R * N * 2;
-    u32x4 wf[KS][TN];
+    constexpr bool W_BLK8 = W_NMAJOR && OES == 2 && TN == 8;    // 8 x 8 blocks (16-byte loads), else 8 x 4 blocks
+    constexpr int NBLK = TN / 4;
+    u32x4 wf[KS][TN];                           // K-major weights and 8 x 8 blocks are loaded into place
+    u32x2 wraw[W_NMAJOR && !W_BLK8 ? NBLK : 1][KS][8];
     if constexpr (W_NMAJOR) {
-        if constexpr (OES == 2 && TN == 8) {
+        if constexpr (W_BLK8) {
             const uint32_t col = (uint32_t)min((a & 3) * 32 + (a >> 2) * 8, N - 8);   // lanes past N recompute a valid block; never stored
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                u32x4 blk[8];
+            for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                 for (int x = 0; x < 8; ++x)
-                    blk[x] = *reinterpret_cast<const u32x4 *>(We + ((uint32_t)(ks * 32 + g * 8 + x) * (uint32_t)N + col) * 2u);
-                transpose8x8_16b(blk, wf[ks]);
-            }
+                    wf[ks][x] = *reinterpret_cast<const u32x4 *>(We + ((uint32_t)(ks * 32 + g * 8 + x) * (uint32_t)N + col) * 2u);
         } else {
-            constexpr int NBLK = TN / 4;
 #pragma unroll
             for (int v = 0; v < NBLK; ++v) {
                 const int start = OES == 4 ? v * 64 + (a & 3) * 16 + (a >> 2) * 4
                                            : ((a >> 1) & 1) * 32 + (a >> 2) * 8 + (a & 1) * 4;
                 const uint32_t col = (uint32_t)min(start, N - 4);
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    u32x2 blk[8];
-                    u32x4 out4[4];
+                for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
                     for (int x = 0; x < 8; ++x)
-                        blk[x] = *reinterpret_cast<const u32x2 *>(We + ((uint32_t)(ks * 32 + g * 8 + x) * (uint32_t)N + col) * 2u);
-                    transpose8x4_16b(blk, out4);
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) wf[ks][v * 4 + c] = out4[c];
-                }
+                        wraw[v][ks][x] = *reinterpret_cast<const u32x2 *>(We + ((uint32_t)(ks * 32 + g * 8 + x) * (uint32_t)N + col) * 2u);
             }
         }
     } else {
@@ -125,24 +129,20 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
         }
     }
 
-    // this lane's pick (row m0 + lane): byte offsets of its source row and of its result row
+    __builtin_amdgcn_sched_barrier(0);          // index and weight loads are issued; nothing below moves above them
+
     uint32_t aoff = 0, coff = 0;
     int state = 0;                              // 0: nothing to store, 1: store the product, 2: store zeros (bad index)
-    {
-        const int m = m0 + lane;
-        const int mm = min(m, Me - 1);
-        const int b = mm / p.K, k = mm - b * p.K;
-        const int64_t pick = ((int64_t)b * p.E + e) * p.K + k;
-        if constexpr (GATHER) {
-            const int32_t t = load_token(p.Ind, p.ind_dtype, pick, p.T);
-            if (t >= 0) aoff = (uint32_t)(((int64_t)b * p.lda_b + (int64_t)t * p.lda_t) * 2);
-            coff = (uint32_t)(pick * N * OES);
-            state = m < Me ? (t >= 0 ? 1 : 2) : 0;
-        } else {
-            aoff = (uint32_t)(pick * R * 2);
-            coff = (uint32_t)(pick * N * OES);
-            state = m < Me ? 1 : 0;
-        }
+    if constexpr (GATHER) {
+        const int64_t t_raw = decode_index_word(t_word, p.Ind, p.ind_dtype, pick);
+        const int32_t t = (t_raw < 0 || t_raw >= (int64_t)p.T) ? -1 : (int32_t)t_raw;
+        if (t >= 0) aoff = (uint32_t)(((int64_t)b_lane * p.lda_b + (int64_t)t * p.lda_t) * 2);
+        coff = (uint32_t)(pick * N * OES);
+        state = m_lane < Me ? (t >= 0 ? 1 : 2) : 0;
+    } else {
+        aoff = (uint32_t)(pick * R * 2);
+        coff = (uint32_t)(pick * N * OES);
+        state = m_lane < Me ? 1 : 0;
     }
 
     // row fragments: lane (a, g) of row tile tq supplies elements [32*ks + 8*g, +8) of row 16*tq + a.  They are
@@ -154,6 +154,28 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
         const uint32_t xo = (uint32_t)__shfl((int)aoff, tq * 16 + (lane >> 2), kWave) + (uint32_t)((lane & 3) * 16);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) xf[tq][ks] = *reinterpret_cast<const u32x4 *>(p.A + xo + ks * 64);
+    }
+    __builtin_amdgcn_sched_barrier(0);          // the row loads are issued before anything waits for weights or rows
+
+    // the weight blocks become operand fragments (register transposes)
+    if constexpr (W_BLK8) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            u32x4 blk[8];
+#pragma unroll
+            for (int x = 0; x < 8; ++x) blk[x] = wf[ks][x];
+            transpose8x8_16b(blk, wf[ks]);
+        }
+    } else if constexpr (W_NMAJOR) {
+#pragma unroll
+        for (int v = 0; v < NBLK; ++v)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                u32x4 out4[4];
+                transpose8x4_16b(wraw[v][ks], out4);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) wf[ks][v * 4 + c] = out4[c];
+            }
     }
 #pragma unroll
     for (int tq = 0; tq < TQ; ++tq)
