@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void dw_kernel(DwParams p)
         }
     };
 
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);    // uniform: what derives from it is scalar work
     const int a = lane & 15, g = lane >> 4;
     const int wave_i0 = wave * (BI / 4);
     f32x4 acc[TI][TJ];

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
     issue_m(0);
 
     // ---------------- MFMA main loop
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int a = lane & 15, g = lane >> 4;
     const int wave_m0 = (wave / WN) * (BM / WM), wave_n0 = (wave % WN) * (BN / WN);
     f32x4 acc[TM][TN];

@@ -143,8 +143,9 @@ static __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind
 // LDS (sh_cnt): (NW + 1) * T + 1 int32.  `rank_tmp` is [B][N] scratch (only touched when a wavefront's
 // slice exceeds 512 picks).  Picks are read at batch element `b`; results are written at batch element
 // `out_b` of seg_off / perm (a caller that keeps them in LDS passes 0 and seg_off = nullptr: the
-// offsets are left in sh_cnt[NW * T ..]).  `after_token_loads` runs right after the token loads have been
-// issued (a caller's own prefetches belong there: the tokens are the sort's critical path).
+// offsets are left in sh_cnt[NW * T ..]).  `after_token_loads` runs once the tokens have been decoded, before the
+// table is built: a caller's own prefetches belong there, they travel while the table is built and the wait
+// for the tokens does not have to cover them.
 struct NoPrefetch { __device__ __forceinline__ void operator()() const {} };
 
 template <class AfterTokenLoads = NoPrefetch>
@@ -154,7 +155,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
                                                AfterTokenLoads after_token_loads = AfterTokenLoads())
 {
     constexpr int MAXC = 8;                             // 64-pick chunks whose tokens (and ranks) are held in registers at a time
-    const int lane = tid & 63, wave = tid >> 6, NW = nthreads >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = nthreads >> 6;
     int32_t *hist = sh_cnt + (size_t)wave * T;          // this wavefront's counters
     int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
     const int64_t base_pick = (int64_t)b * N;           // where this batch element's picks start in Ind
@@ -163,21 +164,33 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
     const int q_begin = wave * slice, q_end = min(N, q_begin + slice);
     const bool in_regs = slice <= MAXC * kWave;
 
-    // tokens of the slice go in flight before anything else
+    // tokens of the slice go in flight before anything else.  Only the loads: decoding a token here would make
+    // each (uniformly guarded) load wait for its own result, one trip to memory after the other
     int32_t tk[MAXC], rk[MAXC];
+    uint64_t tw[MAXC];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        tw[c] = 0;
+        if (in_regs && c * kWave < slice)        // uniform; within the slice the loads are unconditional so that they overlap
+            tw[c] = load_index_word(Ind, ind_dtype, base_pick + min(q_begin + c * kWave + lane, N - 1));
+    }
+
+    for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
+    __syncthreads();
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int q = q_begin + c * kWave + lane;
         int32_t t = -1;
-        if (in_regs && c * kWave < slice)        // uniform; within the slice the loads are unconditional so that they overlap
-            t = load_token(Ind, ind_dtype, base_pick + min(q, N - 1), T);
+        if (in_regs && c * kWave < slice) {
+            const int64_t raw = decode_index_word(tw[c], Ind, ind_dtype, base_pick + min(q, N - 1));
+            t = (raw < 0 || raw >= (int64_t)T) ? -1 : (int32_t)raw;
+        }
         tk[c] = q < q_end ? t : -1;
         rk[c] = 0;
     }
-    after_token_loads();        // whatever else the caller wants in flight while the tokens travel
-
-    for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
-    __syncthreads();
+    // whatever else the caller wants in flight while the table is built.  Only now: the wait for the tokens
+    // would otherwise have to cover these loads too (the counter of outstanding loads holds 63 at most)
+    after_token_loads();
 
     const int nbits = T > 1 ? 32 - __clz(T - 1) : 0;
     const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));

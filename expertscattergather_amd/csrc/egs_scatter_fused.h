@@ -55,7 +55,9 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     constexpr int ES = TT::ES, VEC = TT::VEC;
     constexpr int R = 4 * VEC * KS;
     constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 32-pick) units in flight per wavefront
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // the wavefront index is made known as uniform: units, experts and base addresses derived from it are then
+    // scalar work, and the loads take a scalar base with a per-lane 32-bit offset
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int a = lane & 15, g = lane >> 4;
     // slices of one batch element sit on one XCD (ids congruent modulo 8 share an XCD), so that its
     // rows are fetched from memory once

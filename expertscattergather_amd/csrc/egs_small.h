@@ -64,7 +64,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     const int bid = block - (GATHER ? 0 : p.csr_blocks);
     if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
                          : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: scalar address work
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
     const int m0 = (tile * 4 + wave) * 64;
@@ -297,7 +297,7 @@ __device__ __forceinline__ void dw_small_body(const SmallDwParams &p, const int 
     const int ij = tile - s * (p.i_tiles * p.j_tiles);
     const int it = ij / p.j_tiles, jt = ij - it * p.j_tiles;
     const int i0 = it * 64, j0 = jt * 64;
-    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: scalar address work
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
     const int row_begin = s * p.rows_per_split;
