@@ -175,8 +175,10 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
             tw[c] = load_index_word(Ind, ind_dtype, base_pick + min(q_begin + c * kWave + lane, N - 1));
     }
 
-    for (int i = tid; i < NW * T; i += nthreads) sh_cnt[i] = 0;
-    __syncthreads();
+    // every wavefront clears its own counters: they are private until the prefix below, and a wavefront's LDS
+    // accesses happen in order, so no barrier is needed before it ranks
+    for (int i = lane; i < T; i += kWave) cnt_store(&hist[i], 0);
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int q = q_begin + c * kWave + lane;
@@ -189,8 +191,11 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
         rk[c] = 0;
     }
     // whatever else the caller wants in flight while the table is built.  Only now: the wait for the tokens
-    // would otherwise have to cover these loads too (the counter of outstanding loads holds 63 at most)
-    after_token_loads();
+    // would otherwise have to cover these loads too (the counter of outstanding loads holds 63 at most).
+    // Issuing many loads is bound by the CU's one address path and ranking by VALU issue: the first four
+    // wavefronts prefetch and then rank, the others rank first, so that the two overlap on every SIMD
+    const bool prefetch_first = (wave & 4) == 0;
+    if (prefetch_first) after_token_loads();
 
     const int nbits = T > 1 ? 32 - __clz(T - 1) : 0;
     const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
@@ -232,6 +237,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
             }
         }
     }
+    if (!prefetch_first) after_token_loads();
     __syncthreads();
 
     // per token: counts -> exclusive prefix over wavefronts; total per token
