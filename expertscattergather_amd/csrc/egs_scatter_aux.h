@@ -241,12 +241,17 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
     __syncthreads();
 
     // per token: counts -> exclusive prefix over wavefronts; total per token
+    // (all counts of a token are read before any is overwritten, so that the reads are in flight together)
+    constexpr int kMaxWaves = 16;                       // workgroups have at most 1024 threads
     for (int t = tid; t < T; t += nthreads) {
+        int c[kMaxWaves];
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) c[w] = w < NW ? sh_cnt[(size_t)w * T + t] : 0;
         int run = 0;
-        for (int w = 0; w < NW; ++w) {
-            const int c = sh_cnt[(size_t)w * T + t];
-            sh_cnt[(size_t)w * T + t] = run;
-            run += c;
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) {
+            if (w < NW) sh_cnt[(size_t)w * T + t] = run;
+            run += c[w];
         }
         tok_start[t] = run;
     }
@@ -267,8 +272,9 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
         if (lane == 0) part_total[wave] = running;
         __syncthreads();
         int before = 0, total = 0;
-        for (int w = 0; w < NW; ++w) {
-            const int c = part_total[w];
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) {
+            const int c = w < NW ? part_total[w] : 0;
             if (w < wave) before += c;
             total += c;
         }
