@@ -36,8 +36,7 @@ SIGNATURES = {
     "egs_abi_version": (_i, []),
     "egs_status_string": (ctypes.c_char_p, [_i]),
     "egs_last_hip_error": (ctypes.c_char_p, []),
-    "egs_set_force_generic": (None, [_i]),
-    "egs_set_debug_times": (None, [_vp]),
+    "egs_testing_force_generic": (None, [_i]),       # include/egs_hip_testing.h
     "egs_workspace_bytes": (_sz, [_i, _i, _dp, _i]),
     "egs_gather_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "egs_gemm_scatter": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _i, _vp]),

@@ -3,6 +3,7 @@
 // instantiations compile in parallel with the rest.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stdint.h>
 #include <stdio.h>
 #include <string.h>
@@ -15,7 +16,7 @@
 namespace egs {
 namespace host {
 
-extern bool g_force_generic;        // testing aid: skip the fast paths
+extern std::atomic<bool> g_force_generic;       // testing aid (egs_testing_force_generic): skip the fast paths
 
 int hip_fail(hipError_t err, const char *what);     // records the HIP error text for egs_last_hip_error, returns EGS_ERR_HIP
 const char *last_hip_error();

@@ -2,10 +2,14 @@
 // declared in include/egs_hip.h.  The two template-heavy launch families (tiled rows products,
 // tiled weight gradients) live in egs_rows_launch.hip and egs_dw_launch.hip.
 #include "egs_host.h"
+#include "../../include/egs_hip_testing.h"
 #include "egs_device.h"
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
 #include "egs_scatter_fused.h"
+
+#include <atomic>
+#include <mutex>
 
 using namespace egs;
 using namespace egs::host;
@@ -13,7 +17,7 @@ using namespace egs::host;
 namespace egs {
 namespace host {
 
-bool g_force_generic = false;
+std::atomic<bool> g_force_generic{false};
 static thread_local char g_hip_error_buf[256] = "";
 
 int hip_fail(hipError_t err, const char *what)
@@ -28,7 +32,28 @@ const char *last_hip_error() { return g_hip_error_buf; }
 
 namespace {
 
-unsigned long long *g_dbg_times = nullptr;   // performance debugging: per-wavefront time stamps of the small rows kernel
+constexpr int kMaxDevices = 64;
+
+// A kernel that takes more than 64 KB of dynamic LDS has to be granted it, per device.  One LdsGrant per kernel
+// remembers the largest size granted on each device; growth is serialised so that a smaller request racing
+// with a larger one cannot shrink the grant.
+struct LdsGrant { std::atomic<uint32_t> bytes[kMaxDevices]; };
+std::mutex g_lds_mutex;
+int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *what)
+{
+    if (lds <= 64 * 1024) return EGS_OK;
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return EGS_ERR_UNSUPPORTED;
+    if (grant.bytes[dev].load(std::memory_order_acquire) >= lds) return EGS_OK;
+    std::lock_guard<std::mutex> lock(g_lds_mutex);
+    if (grant.bytes[dev].load(std::memory_order_relaxed) >= lds) return EGS_OK;
+    err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return hip_fail(err, what);
+    grant.bytes[dev].store((uint32_t)lds, std::memory_order_release);
+    return EGS_OK;
+}
 
 bool act_dtype_ok(int d) { return d == EGS_F32 || d == EGS_F16 || d == EGS_BF16; }
 bool ind_dtype_ok(int d) { return d >= EGS_IND_I16 && d <= EGS_IND_U8; }
@@ -251,7 +276,6 @@ bool make_dw_small(const void *Xs, const void *Ys, const void *Ind, void *dW, vo
 template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
 int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
 {
-    j.p.dbg_times = g_dbg_times;
     if (dw != nullptr) {
         hipLaunchKernelGGL((rows_dw_small_kernel<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>), dim3(j.blocks + dw->blocks),
                            dim3(kThreads), j.lds, s, j.p, dw->q, j.blocks);
@@ -329,12 +353,9 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
         while (nw > 1 && csr_count_lds(d->T, nw) > budget) nw >>= 1;
         const size_t lds = csr_count_lds(d->T, nw);
         if (lds <= budget) {
-            static size_t configured = 64 * 1024;
-            if (lds > configured) {
-                hipError_t err = hipFuncSetAttribute((const void *)csr_count_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-                if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(csr_count_kernel)");
-                configured = lds;
-            }
+            static LdsGrant told;
+            const int rc_lds = allow_large_lds((const void *)csr_count_kernel, told, lds, "hipFuncSetAttribute(csr_count_kernel)");
+            if (rc_lds != EGS_OK) return rc_lds;
             hipLaunchKernelGGL(csr_count_kernel, dim3(d->B), dim3(64 * nw), lds, s, Ind, ind_dtype, d->T, (int32_t)N, seg_off, perm, rank_tmp, long_tab);
             EGS_CHECK_LAUNCH("csr_count_kernel");
             return EGS_OK;
@@ -345,12 +366,9 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
     const bool sortable = N >= 1 && NP <= 32768 && (((uint64_t)d->T << QB) <= 0xFFFFFFFFull);
     if (sortable) {
         const size_t lds = (size_t)NP * 4;
-        static size_t configured = 64 * 1024;
-        if (lds > configured) {
-            hipError_t err = hipFuncSetAttribute((const void *)csr_sort_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(csr_sort_kernel)");
-            configured = lds;
-        }
+        static LdsGrant told;
+        const int rc_lds = allow_large_lds((const void *)csr_sort_kernel, told, lds, "hipFuncSetAttribute(csr_sort_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
         int threads = NP / 2;
         if (threads < 64) threads = 64;
         if (threads > 1024) threads = 1024;
@@ -407,29 +425,23 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
 template <class TT, bool W_NMAJOR, int KS>
 int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
 {
-    static size_t configured_plain = 64 * 1024, configured_dw = 64 * 1024;
+    static LdsGrant told_plain, told_dw;        // one pair per template instantiation
     if constexpr (TT::ES != 2) dw = nullptr;            // the small weight gradient exists for 16-bit types only
     if (dw != nullptr) {
       if constexpr (TT::ES == 2) {
         const size_t dw_lds = (size_t)kDwSmallLdsBytes * (kFusedThreads / kThreads);       // one 16 KB tile per wavefront
         const size_t need = lds > dw_lds ? lds : dw_lds;
-        if (need > configured_dw) {
-            hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_dw_kernel<TT, W_NMAJOR, KS>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)need);
-            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_dw_kernel)");
-            configured_dw = need;
-        }
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_dw_kernel<TT, W_NMAJOR, KS>, told_dw, need,
+                                           "hipFuncSetAttribute(scatter_fused_dw_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_dw_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dw->blocks), dim3(kFusedThreads), need, s, p,
                            dw->q, blocks);
         dw->done = true;
       }
     } else {
-        if (lds > configured_plain) {
-            hipError_t err = hipFuncSetAttribute((const void *)scatter_fused_kernel<TT, W_NMAJOR, KS>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (err != hipSuccess) return hip_fail(err, "hipFuncSetAttribute(scatter_fused_kernel)");
-            configured_plain = lds;
-        }
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_kernel<TT, W_NMAJOR, KS>, told_plain, lds,
+                                           "hipFuncSetAttribute(scatter_fused_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     }
     EGS_CHECK_LAUNCH("scatter_fused_kernel");
@@ -743,8 +755,7 @@ const char *egs_status_string(int status)
 
 const char *egs_last_hip_error(void) { return last_hip_error(); }
 
-void egs_set_force_generic(int on) { g_force_generic = on != 0; }
-void egs_set_debug_times(void *buf) { g_dbg_times = (unsigned long long *)buf; }
+void egs_testing_force_generic(int on) { g_force_generic.store(on != 0); }
 
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
 {

@@ -45,19 +45,26 @@ static __global__ __launch_bounds__(kThreads) void quantize_rows_e4m3_kernel(Qua
     const int64_t b = row / p.T, t = row - b * p.T;
     const char *src = p.X + (b * p.ldx_b + t * p.ldx_t) * 2;
     const int chunks = p.I >> 3;
-    float amax = 0.f;
+    // max|x| over the row as an integer maximum of the magnitude bits: for non-negative floats the bit patterns
+    // order like the values, infinities sort above every finite value and NaNs above the infinities, so a NaN
+    // anywhere in the row survives the reduction (fmaxf would drop it)
+    uint32_t amax_bits = 0u;
     for (int c = lane; c < chunks; c += 64) {
         const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (size_t)c * 16);
 #pragma unroll
         for (int x = 0; x < 4; ++x) {
-            amax = fmaxf(amax, fabsf(bits_f32(v[x] << 16)));
-            amax = fmaxf(amax, fabsf(bits_f32(v[x] & 0xffff0000u)));
+            amax_bits = max(amax_bits, (v[x] << 16) & 0x7fffffffu);
+            amax_bits = max(amax_bits, v[x] & 0x7fff0000u);
         }
     }
 #pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) amax = fmaxf(amax, __shfl_xor(amax, m));
-    const float scale = amax > 0.f ? amax / kE4M3Max : 1.0f;
-    const float inv = 1.0f / scale;
+    for (int m = 32; m >= 1; m >>= 1) amax_bits = max(amax_bits, (uint32_t)__shfl_xor((int)amax_bits, m));
+    const float amax = bits_f32(amax_bits);
+    // a row that holds a NaN or an infinity gets a NaN scale: every product that uses the row comes out NaN,
+    // as it does in unquantised arithmetic (the quantised values themselves are then meaningless)
+    const bool finite = amax_bits < 0x7f800000u;
+    const float scale = !finite ? bits_f32(0x7fc00000u) : (amax > 0.f ? amax / kE4M3Max : 1.0f);
+    const float inv = finite ? 1.0f / scale : 0.f;
     if (lane == 0) p.xs[row] = scale;
     char *dst = p.Xq + row * p.I;
     for (int c = lane; c < chunks; c += 64) {

@@ -569,8 +569,15 @@ __device__ __forceinline__ void segment_sum_long_body(const SegSumParams &sp, co
             __hip_atomic_store(part + iv, acc[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0);      // this thread's partial-row stores have completed
-    __syncthreads();                    // ... and so have everybody else's, before the arrival is counted
+    // Hand-off to the workgroup that arrives last.  The partial-row stores above are agent-scope atomic stores:
+    // they bypass this XCD's non-coherent cache state and are acknowledged by the memory side.  The wait below
+    // (stores count on the vector-memory counter) returns once this thread's stores have been acknowledged, and
+    // as a volatile statement with a memory clobber it also keeps the compiler from moving any of them past it.
+    // The barrier then orders every thread's acknowledged stores before thread 0's arrival count, which is an
+    // agent-scope read-modify-write at the same memory side; a workgroup that observes nch - 1 there therefore
+    // reads, with agent-scope loads that also go to the memory side, rows that are complete.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     if (tid == 0)
         sh_last = (__hip_atomic_fetch_add(&rec[3], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nch - 1) ? 1 : 0;
     __syncthreads();

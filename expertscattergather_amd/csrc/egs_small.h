@@ -41,7 +41,6 @@ struct SmallRowsParams {
     // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
     int32_t csr_blocks;
     int32_t *seg_off, *perm, *rank_tmp, *long_tab;
-    unsigned long long *dbg_times;   // optional [grid*4][2] wall-clock stamps per wavefront (performance debugging)
 };
 
 // Requirements (checked by the launcher): 2-byte elements, R == 32*KS, N % 8 == 0,
@@ -70,7 +69,6 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     const int m0 = (tile * 4 + wave) * 64;
     if (m0 >= Me) return;                       // no barriers below: a wave may leave alone
     const int N = p.N;
-    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)block * 4 + wave) * 2] = wall_clock64();
 
     // Order of the loads.  Loads return in order, and the long chain is index -> row.  So the index load goes
     // first, the weight loads follow in the shadow of its latency, and the row loads are issued as soon as the
@@ -241,7 +239,6 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
             }
         }
     }
-    if (p.dbg_times != nullptr && lane == 0) p.dbg_times[((size_t)block * 4 + wave) * 2 + 1] = wall_clock64();
 }
 
 template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>

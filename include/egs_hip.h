@@ -8,6 +8,9 @@
  *
  * Conventions for every entry point
  *   - returns EGS_OK (0) or a negative egs_status; never throws, never synchronises;
+ *   - thread-safe and re-entrant: the library keeps no mutable state except once-per-device
+ *     set-up flags; it launches on
+ *     the calling thread's current device;
  *   - all tensor pointers are device pointers, borrowed until the enqueued work completes;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = default stream);
  *   - arguments are validated before any HIP call, so bad arguments are reported even on a
@@ -16,6 +19,10 @@
  *     from egs_workspace_bytes();
  *   - tensors are dense row-major ([B,T,I] sources may carry explicit batch/token strides,
  *     inner stride 1);  Ind is [B,E,K] of int16/int32/int64/uint8 and is never written;
+ *   - Ind is read through aligned 8-byte windows: the 8-byte aligned words that contain its first
+ *     and its last element must lie inside the allocation.  Any buffer that starts at an address
+ *     hipMalloc (or an allocator that rounds to 8 bytes or more, such as torch's) returned, or at
+ *     an element offset into one, satisfies this;
  *   - a pick whose index is outside [0,T) contributes nothing (gather writes a zero row,
  *     scatter and dW skip it); egs_validate_indices() reports such picks.
  */
@@ -91,15 +98,6 @@ int egs_abi_version(void);
 const char *egs_status_string(int status);
 /* text of the last HIP error seen by the calling thread ("" if none) */
 const char *egs_last_hip_error(void);
-
-/* Testing aid: non-zero routes every call through the general tiled kernels, skipping the
- * specialised small-expert kernels (both must give results within the same tolerances). */
-void egs_set_force_generic(int on);
-
-/* Performance-debugging aid: when `buf` is non-NULL (device memory, 2 x uint64 per wavefront of
- * the launch, zero-filled by the caller) the small-expert rows kernel stamps the 100 MHz wall
- * clock at each wavefront's start and end.  NULL switches it off. */
-void egs_set_debug_times(void *buf);
 
 /* bytes of scratch the op needs for these sizes (0 is a valid answer).
  * `mode` is an egs_scatter_mode and only matters for ops that scatter. */

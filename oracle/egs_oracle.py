@@ -283,12 +283,18 @@ def float_to_fp8_e4m3fn(x) -> np.ndarray:
 
 def quantize_rows_e4m3(X):
     """Per-row e4m3 quantisation of X[..., I] in float32 arithmetic: scale = max|row| / 448 (1 for a zero
-    row), q = encode(clamp(x * (1 / scale), -448, 448)).  Returns (bytes [..., I], scale [...])."""
+    row, NaN for a row with a non-finite element), q = encode(clamp(x * (1 / scale), -448, 448)).
+    Returns (bytes [..., I], scale [...])."""
     X = np.asarray(X, dtype=np.float32)
-    amax = np.abs(X).max(axis=-1)
+    finite = np.isfinite(X).all(axis=-1)
+    Xf = np.where(finite[..., None], X, np.float32(0.0))
+    amax = np.abs(Xf).max(axis=-1)
     scale = np.where(amax > 0, amax / np.float32(448.0), np.float32(1.0)).astype(np.float32)
     inv = (np.float32(1.0) / scale).astype(np.float32)
-    y = np.clip((X * inv[..., None]).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    y = np.clip((Xf * inv[..., None]).astype(np.float32), np.float32(-448.0), np.float32(448.0))
+    # a row that holds a NaN or an infinity cannot be represented: its scale is NaN, so that every product
+    # using the row is NaN as in unquantised arithmetic; its bytes are unspecified (zeros here)
+    scale = np.where(finite, scale, np.float32(np.nan)).astype(np.float32)
     return float_to_fp8_e4m3fn(y), scale
 
 

@@ -87,9 +87,9 @@ SMALL_SHAPES = [
 @pytest.fixture(params=[False, True], ids=["fastpaths", "generic"])
 def force_generic(request):
     from expertscattergather_amd import _abi
-    _abi.lib().egs_set_force_generic(1 if request.param else 0)
+    _abi.lib().egs_testing_force_generic(1 if request.param else 0)
     yield request.param
-    _abi.lib().egs_set_force_generic(0)
+    _abi.lib().egs_testing_force_generic(0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])

@@ -198,3 +198,10 @@ def test_fp8_encoder_and_row_quantiser_match_torch():
     # a quantised row reproduces the row to e4m3 accuracy: |x - dequant| <= 2^-4 |x| + half a subnormal step
     deq = O.fp8_e4m3fn_to_float(q) * xs[..., None]
     assert (np.abs(deq - X.float().numpy()) <= 2.0 ** -4 * np.abs(X.float().numpy()) + xs[..., None] * 2.0 ** -10).all()
+    # rows with a NaN or an infinity: NaN scale (every product of the row is NaN, as in unquantised arithmetic);
+    # the other rows are untouched
+    Xn = X.float().numpy().copy()
+    Xn[0, 0, 5] = np.nan; Xn[3, 2, 0] = np.inf; Xn[6, 4, 63] = -np.inf
+    q2, xs2 = O.quantize_rows_e4m3(Xn)
+    bad = np.zeros(xs.shape, dtype=bool); bad[0, 0] = bad[3, 2] = bad[6, 4] = True
+    assert np.isnan(xs2[bad]).all() and np.array_equal(xs2[~bad], xs[~bad]) and np.array_equal(q2[~bad], q[~bad])
