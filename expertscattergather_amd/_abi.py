@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(HERE, "libegs_hip.so")
 EGS_OK = 0
 EGS_ERR_BAD_DTYPE = -3
 EGS_ERR_HIP = -8
+EGS_ERR_SCRATCH_LIMIT = -11
+BUILTIN_SCRATCH_BYTES = 16 << 20
 F32, F16, BF16, FP8_E4M3 = 0, 1, 2, 3
 IND_I16, IND_I32, IND_I64, IND_U8 = 0, 1, 2, 3
 W_EIJ, W_EJI = 0, 1
@@ -41,6 +43,7 @@ SIGNATURES = {
     "egs_gather_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "egs_gemm_scatter": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _i, _vp]),
     "egs_dw": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
+    "egs_dw_builtin_scratch": (_i, [_vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "egs_gather_gemm_fp8act_workspace_bytes": (_sz, [_dp]),
     "egs_gather_gemm_fp8act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _vp]),
     "egs_expert_gather_forward": (_i, [_vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _vp]),

@@ -32,7 +32,17 @@ const char *last_hip_error() { return g_hip_error_buf; }
 
 namespace {
 
+// ------------------------------------------------------------------------------ built-in scratch
+// Device memory that exists from the moment the library's code object is loaded, for the one entry
+// point that serves callers which cannot allocate (egs_dw_builtin_scratch).  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends.
+// The array's name is only a host-side handle: host code never passes it to a kernel or a copy.  The
+// device address is looked up once per device (with that device current) and kept.
+static __device__ __align__(256) unsigned char scratch[EGS_BUILTIN_SCRATCH_BYTES];
+
 constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];              // per device: address of that device's copy of `scratch`
 
 // A kernel that takes more than 64 KB of dynamic LDS has to be granted it, per device.  One LdsGrant per kernel
 // remembers the largest size granted on each device; growth is serialised so that a smaller request racing
@@ -52,6 +62,24 @@ int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *wha
     err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return hip_fail(err, what);
     grant.bytes[dev].store((uint32_t)lds, std::memory_order_release);
+    return EGS_OK;
+}
+
+int builtin_scratch_ptr(void **out)
+{
+    int dev = -1;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return hip_fail(err, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return EGS_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        err = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return hip_fail(err, "hipGetSymbolAddress(scratch)");
+        if (ptr == nullptr) return EGS_ERR_HIP;
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
     return EGS_OK;
 }
 
@@ -749,6 +777,7 @@ const char *egs_status_string(int status)
     case EGS_ERR_HIP: return "HIP runtime error";
     case EGS_ERR_UNSUPPORTED: return "unsupported dtype combination";
     case EGS_ERR_BAD_STRIDE: return "source stride smaller than its row";
+    case EGS_ERR_SCRATCH_LIMIT: return "sizes need more scratch than the built-in buffer holds (EGS_BUILTIN_SCRATCH_BYTES)";
     default: return "unknown status";
     }
 }
@@ -800,6 +829,31 @@ int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
                          ind_dtype, dw_layout);
     if (rc != EGS_OK) return rc;
     return dw_impl(Xsrc, Ysrc, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout,
+                   (hipStream_t)stream);
+}
+
+int egs_dw_builtin_scratch(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW, const egs_dims *d,
+                           int64_t ldx_b, int64_t ldx_t,
+                           int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream)
+{
+    int rc = check_dims(d);
+    if (rc != EGS_OK) return rc;
+    if (!act_dtype_ok(act_dtype)) return EGS_ERR_BAD_DTYPE;
+    const size_t need = plan_dw(d, act_dtype).bytes;
+    if (need > (size_t)EGS_BUILTIN_SCRATCH_BYTES) return EGS_ERR_SCRATCH_LIMIT;
+    // the remaining checks are those of egs_dw; the stand-in address only has to look like a valid workspace
+    rc = validate_dw(Xsrc, Ysrc, Ind, dW, need > 0 ? (const void *)(uintptr_t)256 : nullptr, need, d, ldx_b, ldx_t, act_dtype,
+                     out_dtype, ind_dtype, dw_layout);
+    if (rc != EGS_OK) return rc;
+    if ((size_t)d->E * d->I * d->J == 0) return EGS_OK;
+    void *ws = nullptr;
+    if (need > 0) {
+        rc = builtin_scratch_ptr(&ws);
+        if (rc != EGS_OK) return rc;
+    }
+    // the partial sums of every split are written before the second pass reads them: nothing in the
+    // buffer has to start at zero
+    return dw_impl(Xsrc, Ysrc, Ind, dW, ws, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout,
                    (hipStream_t)stream);
 }
 

@@ -9,7 +9,7 @@
  * Conventions for every entry point
  *   - returns EGS_OK (0) or a negative egs_status; never throws, never synchronises;
  *   - thread-safe and re-entrant: the library keeps no mutable state except once-per-device
- *     set-up flags; it launches on
+ *     set-up flags (and the built-in buffer of egs_dw_builtin_scratch, see there); it launches on
  *     the calling thread's current device;
  *   - all tensor pointers are device pointers, borrowed until the enqueued work completes;
  *   - work is enqueued on `stream` (a hipStream_t passed as void*, NULL = default stream);
@@ -49,7 +49,8 @@ typedef enum egs_status {
     EGS_ERR_ALIGNMENT = -7,
     EGS_ERR_HIP = -8,           /* a HIP runtime call failed; see egs_last_hip_error() */
     EGS_ERR_UNSUPPORTED = -9,
-    EGS_ERR_BAD_STRIDE = -10
+    EGS_ERR_BAD_STRIDE = -10,
+    EGS_ERR_SCRATCH_LIMIT = -11 /* egs_dw_builtin_scratch: the sizes need more than EGS_BUILTIN_SCRATCH_BYTES */
 } egs_status;
 
 /* element types; 0..2 are the reference's dtype ids (egs/triton_kernels.py:15-23) */
@@ -135,6 +136,23 @@ int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
            void *workspace, size_t workspace_bytes, const egs_dims *d,
            int64_t ldx_b, int64_t ldx_t,
            int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream);
+
+/* egs_dw for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference, whose launchers allocate
+ * with torch on every call (egs/triton_kernels.py:408-409, :491-492).
+ * Same arguments, kernels and results (bit for bit) as egs_dw, minus the workspace: the fp32 partial
+ * sums of the split reduction live in a buffer of EGS_BUILTIN_SCRATCH_BYTES that is part of the
+ * library's device image (every GPU the library runs on holds one until the process ends).  The call
+ * allocates and frees nothing; the buffer's device address is looked up the first time the entry point
+ * runs on a device, so make that first call outside graph capture.
+ * Sizes whose partial sums (egs_workspace_bytes(EGS_OP_DW, ...)) exceed the buffer are rejected with
+ * EGS_ERR_SCRATCH_LIMIT before anything is enqueued.
+ * All calls on one GPU share that GPU's buffer: calls that may overlap in time (different streams,
+ * different threads) race on it; serialise them, or use egs_dw with workspaces of their own. */
+#define EGS_BUILTIN_SCRATCH_BYTES (16u << 20)
+int egs_dw_builtin_scratch(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW, const egs_dims *d,
+                           int64_t ldx_b, int64_t ldx_t,
+                           int act_dtype, int out_dtype, int ind_dtype, int dw_layout, void *stream);
 
 /* Inference variant of the gather with fp8 weights AND fp8 activations, on the fp8 matrix instruction:
  *   Y[b,e,k,j] = xs[b,t] * w_scale[e,j] * sum_i Xq[b,t,i] * Wq(e,i,j),   t = Ind[b,e,k],

@@ -41,7 +41,7 @@ def test_version_and_status_strings(lib):
     assert lib.egs_abi_version() == _abi.ABI_VERSION == 1
     assert lib.egs_status_string(0) == b"ok"
     assert lib.egs_status_string(_abi.EGS_ERR_BAD_DTYPE) == b"Unknown dtype"
-    for code in range(-10, 0):
+    for code in range(-11, 0):
         assert lib.egs_status_string(code) not in (b"", b"unknown status")
     assert lib.egs_status_string(-99) == b"unknown status"
     assert lib.egs_last_hip_error() == b""
@@ -89,6 +89,22 @@ def test_argument_validation_needs_no_gpu(lib):
     empty = _abi.Dims(0, 8, 3, 4, 16, 8)
     assert g(None, None, None, None, None, empty, 0, 0, 2, 2, 2, 0, None) == 0
     assert sc(None, None, None, None, None, 0, empty, 2, 2, 1, 0, None) == 0
+
+
+def test_builtin_scratch_entry_point_checks_sizes_first(lib):
+    # sizes whose partial sums do not fit the built-in buffer are refused before any pointer is looked at
+    big = _abi.Dims(16, 512, 4, 256, 1024, 1024)
+    assert lib.egs_workspace_bytes(_abi.OP_DW, 0, big, _abi.BF16) > _abi.BUILTIN_SCRATCH_BYTES
+    f = lib.egs_dw_builtin_scratch
+    p = 0x1000
+    assert f(p, p, p, p, big, 512 * 1024, 1024, 2, 2, 2, 0, None) == _abi.EGS_ERR_SCRATCH_LIMIT == -11
+    d = _abi.Dims(2, 8, 3, 4, 16, 8)
+    assert f(p, p, p, None, d, 128, 16, 2, 2, 2, 0, None) == -1               # null output
+    assert f(p, p, p, p, d, 128, 16, 7, 2, 2, 0, None) == -3                  # unknown dtype
+    assert f(p, p, p, p, d, 128, 16, 2, 2, 2, 5, None) == -4                  # unknown layout
+    text = open(HEADER).read()
+    m = re.search(r"#define\s+EGS_BUILTIN_SCRATCH_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", text)
+    assert m and int(m.group(1)) << int(m.group(2)) == _abi.BUILTIN_SCRATCH_BYTES
 
 
 def test_workspace_sizes_are_consistent(lib):
