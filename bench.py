@@ -51,7 +51,10 @@ def parse_args():
     ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
     ap.add_argument("--cold", action="store_true", help="also time each kernel with the caches flushed between launches")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="only launch a 64 MiB device copy (3x) and the dominant kernel (5x), for rocprofv3 --pmc runs")
+                    help="only launch a 64 MiB device copy (3x) and one entry point of the path (5x), for rocprofv3 --pmc runs")
+    ap.add_argument("--probe-kernel", default="gather", choices=["gather", "scatter", "dw", "scatter_bwd", "gather_bwd"],
+                    help="which entry point --pmc-probe launches: gather forward, scatter forward, the stand-alone weight "
+                         "gradient, or one of the two backward calls (each shares its launch with a weight gradient)")
     return ap.parse_args()
 
 
@@ -84,11 +87,28 @@ def main():
             dst.copy_(src)
         if args.config == "C5":     # the configuration's own weights: e4m3 bytes and fp32 scales
             Wq_p, scale_p = (t.to(dev) for t in wl.quantize_fp8_weights(inp["Wg"].float()))
+        Yp = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32) if args.config != "C5" else None
+        if args.probe_kernel == "dw":
+            dWp = torch.empty_like(Wg)
+            dp = _abi.Dims(B, T, E, K, I, J)
+            dtp = hk.dtype_to_type_id(cfg.dtype)
+            wsb = max(_abi.lib().egs_workspace_bytes(_abi.OP_DW, 0, dp, dtp), 256)
+            wsp = torch.empty(wsb, dtype=torch.uint8, device=dev)
         for _ in range(5):
             if args.config == "C5":
                 hk.expert_gather_fp8w_forward(X, Wq_p, scale_p, Ind)
-            else:
+            elif args.probe_kernel == "gather":
                 hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+            elif args.probe_kernel == "scatter":
+                hk.expert_scatter_forward_call(Yp, Ws, Ind, T, torch.float32)
+            elif args.probe_kernel == "scatter_bwd":
+                hk.expert_scatter_backward_call(Yp, Ws, Ind, dOut, torch.float32)
+            elif args.probe_kernel == "gather_bwd":
+                hk.expert_gather_backward_call(X, Wg, Ind, Yp, torch.float32)
+            else:
+                rc = _abi.lib().egs_dw(X.data_ptr(), Yp.data_ptr(), Ind.data_ptr(), dWp.data_ptr(), wsp.data_ptr(), wsb, dp,
+                                       T * I, I, dtp, dtp, _abi.IND_I64, _abi.W_EIJ, torch.cuda.current_stream().cuda_stream)
+                assert rc == 0
         torch.cuda.synchronize()
         print(json.dumps({"pmc_probe": True, "copy_bytes_read": 64 << 20, "copy_bytes_written": 64 << 20}))
         return

@@ -1,0 +1,279 @@
+// Weight gradient of small experts in ONE pass, no split of the picks and therefore no partial sums
+// and no second launch:
+//
+//   dW(e, i, j) = sum over all picks m = (b, k) of expert e of  Xs[b, Ind[b,e,k], i] * Ys[b, e, k, j]
+//
+// A workgroup owns a 32 x TJ tile of dW(e) (TJ = 32 or 64) and reduces ALL of the expert's picks; with
+// E * (I/32) * (J/TJ) workgroups (256 or 128 at the reference's default shape E32 I128 J64) the device is busy
+// without splitting the reduction.  Its wavefronts take contiguous parts of the picks, each accumulating the
+// whole tile, and are summed through LDS in wavefront order (fixed order -> bitwise reproducible, no atomics).
+// What bounds the kernel is the rate at which a CU can send requests to its L2 (about one per 2.4 cycles,
+// whatever their size up to a 128-byte line): 64 columns on the Ys side make that side's requests full lines.
+//
+// Both operands are "reduction-strided" in memory (a pick selects a row, the output index runs along it),
+// the opposite of what the matrix instruction wants (per lane: 8 consecutive picks of one column).  Per
+// 32-pick step a wavefront fetches the 64-byte pieces of 32 gathered Xs rows and the 64- or 128-byte pieces of
+// 32 Ys rows with 16-byte buffer loads (adjacent lanes take adjacent chunks of a pick's piece: one access per
+// row), keeps a whole chunk of picks in flight in registers, drops each step into a wavefront-private LDS tile
+// as [pick][column] and reads the fragments back with the LDS transpose read.  No barrier in the main loop.  Row byte offsets come from a table in LDS that the wavefront decodes
+// from Ind one chunk ahead; picks that do not exist (bad index, ragged end) get an offset outside the buffer
+// descriptor and arrive as zeros on both sides.
+//
+// Replaces the reference's expert_gather_scatter_dW_kernel (egs/triton_kernels.py:261-356), which reduces
+// over the batch only and adds the K partial tiles with atomics in the output type.
+#pragma once
+#include "egs_device.h"
+
+namespace egs {
+
+struct DwTileParams {
+    const char *Xs;         // [B,T,I] rows, strides (ldx_b, ldx_t, 1) in elements; x_bytes < 2 GiB
+    const char *Ys;         // [B,E,K,J] dense; y_bytes < 2 GiB
+    const void *Ind;
+    char *dW;               // [E,I,J] or [E,J,I] in out_dtype
+    int32_t B, T, E, K, I, J;       // I % 8 == 0, J % 8 == 0
+    int64_t ldx_b, ldx_t;
+    int32_t ind_dtype;
+    int32_t i_tiles, j_tiles;       // 32-column tiles of I and of J
+    int32_t out_dtype, dw_layout;
+    uint32_t x_bytes, y_bytes;
+};
+
+// picks whose rows a wavefront keeps in flight at a time (registers: 16 or 24 per 32-pick step)
+__host__ __device__ constexpr int dw_tile_chunk(int TJ) { return TJ == 32 ? 256 : 128; }
+// per wavefront: row-offset tables of two chunks (Xs and Ys side) + two staging tiles (Xs piece 2 KB, Ys piece TJ * 64 bytes)
+__host__ __device__ constexpr int dw_tile_lds_per_wave(int TJ) { return 2 * 2 * dw_tile_chunk(TJ) * 4 + 2 * (2048 + TJ * 64); }
+__host__ __device__ constexpr size_t dw_tile_lds(int waves, int TJ = 32) { return (size_t)waves * dw_tile_lds_per_wave(TJ); }
+
+__device__ __forceinline__ u32x4 buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff)
+{
+    return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff, 0, 0));
+}
+
+// Requirements (checked by the launcher): 2-byte elements, I % 8 == 0, J % 8 == 0, rows of Xs and Ys 16-byte
+// aligned, both tensors below 2 GiB, dW 16-byte aligned, T >= 1; j_tiles counts TJ-column tiles.
+// `smem`: dw_tile_lds(NW, TJ) bytes, 16-byte aligned.
+template <class TT, int NW, int TJ = 32>
+__device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int block, char *smem)
+{
+    static_assert(TT::ES == 2, "16-bit element types");
+    static_assert(TJ == 32 || TJ == 64, "Ys-side tile width");
+    constexpr int CH = dw_tile_chunk(TJ), NS = CH / 32;
+    constexpr int kLdsPerWave = dw_tile_lds_per_wave(TJ);
+    constexpr int YB = TJ * 2;                  // bytes of a Ys piece
+    constexpr int YL = YB / 16;                 // lanes per Ys piece (4 or 8)
+    constexpr int YN = 32 * YL / 64;            // Ys loads per step (2 or 4), 64 / YL picks each
+    constexpr int STG = 2048 + 32 * YB;         // bytes of a staging tile
+    constexpr int NY = TJ / 16;                 // 16-column groups on the Ys side
+    int e, tile;
+    const int tiles_per_e = p.i_tiles * p.j_tiles;
+    if (!decode_expert_tile(block, tiles_per_e, p.E, e, tile)) return;
+    const int it = tile / p.j_tiles, jt = tile - it * p.j_tiles;
+    const int i0 = it * 32, j0 = jt * TJ;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int a = lane & 15, g = lane >> 4;
+    const int Me = p.B * p.K;
+    const int per_wave = ((Me + NW - 1) / NW + 31) & ~31;
+    const int w_begin = min(Me, wave * per_wave), w_end = min(Me, w_begin + per_wave);
+    const int nchunks = (w_end - w_begin + CH - 1) / CH;
+
+    char *mine = smem + wave * kLdsPerWave;
+    uint32_t *tab = reinterpret_cast<uint32_t *>(mine);         // [2][x: CH | y: CH]
+    char *stage = mine + 2 * 2 * CH * 4;                        // [2][Xs piece 2 KB | Ys piece 32 * YB]
+
+    const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p.Xs), 0, (int)p.x_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_y = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p.Ys), 0, (int)p.y_bytes, 0x00020000);
+
+    // this lane's share of a step: Xs picks (lane >> 2) and 16 + (lane >> 2), 16-byte chunk (lane & 3) of the tile's
+    // columns; Ys picks (lane / YL) + (64 / YL) * h, chunk lane % YL
+    const int xc = i0 + (lane & 3) * 8, yc = j0 + (lane % YL) * 8;
+    const uint32_t xcol = xc < p.I ? (uint32_t)xc * 2u : kVoffInvalid;
+    const uint32_t ycol = yc < p.J ? (uint32_t)yc * 2u : kVoffInvalid;
+
+    uint64_t iw[CH / 64];
+    auto pick_of = [&](int c, int u, int &m, int &b) -> int64_t {
+        m = w_begin + c * CH + u * 64 + lane;
+        const int mm = min(m, Me - 1);
+        b = mm / p.K;
+        return ((int64_t)b * p.E + e) * p.K + (mm - b * p.K);
+    };
+    auto load_idx = [&](int c) {
+#pragma unroll
+        for (int u = 0; u < CH / 64; ++u) {
+            int m, b;
+            const int64_t pick = pick_of(c, u, m, b);
+            iw[u] = load_index_word(p.Ind, p.ind_dtype, pick);
+        }
+    };
+    auto store_tab = [&](int c) {
+        uint32_t *t = tab + (c & 1) * 2 * CH;
+#pragma unroll
+        for (int u = 0; u < CH / 64; ++u) {
+            int m, b;
+            const int64_t pick = pick_of(c, u, m, b);
+            const int64_t raw = decode_index_word(iw[u], p.Ind, p.ind_dtype, pick);
+            const bool live = m < w_end && raw >= 0 && raw < (int64_t)p.T;
+            t[u * 64 + lane] = live ? (uint32_t)(((int64_t)b * p.ldx_b + raw * p.ldx_t) * 2) : kVoffInvalid;
+            t[CH + u * 64 + lane] = live ? (uint32_t)(pick * p.J * 2) : kVoffInvalid;
+        }
+    };
+
+    u32x4 rx[NS][2], ry[NS][YN];
+    auto issue = [&](int c, int s) {
+        const uint32_t *t = tab + (c & 1) * 2 * CH;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t xo = t[s * 32 + h * 16 + (lane >> 2)];
+            rx[s][h] = buffer_load16(rs_x, (xo == kVoffInvalid || xcol == kVoffInvalid) ? kVoffInvalid : xo + xcol);
+        }
+#pragma unroll
+        for (int h = 0; h < YN; ++h) {
+            const uint32_t yo = t[CH + s * 32 + h * (64 / YL) + lane / YL];
+            ry[s][h] = buffer_load16(rs_y, (yo == kVoffInvalid || ycol == kVoffInvalid) ? kVoffInvalid : yo + ycol);
+        }
+    };
+
+    f32x4 acc[2][NY];
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int y = 0; y < NY; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // fragment addresses inside a piece ([32 picks][64 or YB bytes]): the lane points at pick 8 g + 4 h + a / 4 and the
+    // four columns 4 (a % 4) of a 16-column group, and receives column a of picks 8 g + 4 h .. + 3
+    const int at0 = (g * 8 + (a >> 2)) * 64 + (a & 3) * 8, at1 = at0 + 4 * 64;
+    const int yat0 = (g * 8 + (a >> 2)) * YB + (a & 3) * 8, yat1 = yat0 + 4 * YB;
+    const int wr = (lane >> 2) * 64 + (lane & 3) * 16;
+    const int ywr = (lane / YL) * YB + (lane % YL) * 16;
+    // A step goes registers -> LDS tile (stage_write), LDS tile -> fragments (stage_read), fragments -> MFMAs.  The
+    // loop is software-pipelined: the fragments of step s are requested first, then the registers of step s+1 are
+    // dropped into the other tile (and refilled from the next chunk), then the MFMAs of step s run - so the LDS
+    // round trip of one step hides behind the work of its neighbours.
+    auto stage_write = [&](int s) {
+        char *st = stage + (s & 1) * STG;
+#pragma unroll
+        for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4 *>(st + h * 1024 + wr) = rx[s][h];
+#pragma unroll
+        for (int h = 0; h < YN; ++h) *reinterpret_cast<u32x4 *>(st + 2048 + h * 1024 + ywr) = ry[s][h];
+    };
+    auto stage_read = [&](int s, u32x4 (&pf)[2], u32x4 (&qf)[NY]) {
+        const char *st = stage + (s & 1) * STG;
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            const u32x2 lo = lds_read_tr16(st + at0 + x * 32), hi = lds_read_tr16(st + at1 + x * 32);
+            pf[x] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+#pragma unroll
+        for (int y = 0; y < NY; ++y) {
+            const u32x2 lo = lds_read_tr16(st + 2048 + yat0 + y * 32), hi = lds_read_tr16(st + 2048 + yat1 + y * 32);
+            qf[y] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+        }
+    };
+    auto chunk_len = [&](int c) { return c < nchunks ? min(CH, w_end - w_begin - c * CH) : 0; };
+
+    if (nchunks > 0) {
+        load_idx(0);
+        store_tab(0);
+        if (nchunks > 1) { load_idx(1); }
+        const int len0 = chunk_len(0);
+#pragma unroll
+        for (int s = 0; s < NS; ++s)
+            if (s * 32 < len0) issue(0, s);
+        if (nchunks > 1) { store_tab(1); }
+        if (nchunks > 2) load_idx(2);
+        stage_write(0);
+        if (nchunks > 1) issue(1, 0);
+    }
+    for (int c = 0; c < nchunks; ++c) {
+        const int len = chunk_len(c), len1 = chunk_len(c + 1), len2 = chunk_len(c + 2);
+        // the table of chunk c+2 replaces that of chunk c, whose loads have all been issued; its index words were
+        // requested a chunk ago
+        if (len2 > 0) store_tab(c + 2);
+        if (c + 3 < nchunks) load_idx(c + 3);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (s * 32 < len) {
+                u32x4 pf[2], qf[NY];
+                stage_read(s, pf, qf);
+                __builtin_amdgcn_sched_barrier(0);
+                if (s + 1 < NS && (s + 1) * 32 < len) {
+                    stage_write(s + 1);
+                    if ((s + 1) * 32 < len1) issue(c + 1, s + 1);
+                } else if (len1 > 0) {                  // last step of the chunk: the next chunk's first step
+                    stage_write(0);
+                    if (len2 > 0) issue(c + 2, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int x = 0; x < 2; ++x)
+#pragma unroll
+                    for (int y = 0; y < NY; ++y) mma_chunk<TT>(acc[x][y], qf[y], pf[x]);
+            }
+        }
+    }
+    __syncthreads();                                    // every wavefront is done with its tables and staging tiles
+
+    // lane (a, g) holds dW rows i0 + 16 x + a, columns j0 + 16 y + 4 g .. + 3
+    float *red = reinterpret_cast<float *>(smem);       // [NW][32 i][TJ j]
+    static_assert(32 * TJ * 4 <= kLdsPerWave, "reduction buffer fits");
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int y = 0; y < NY; ++y)
+            *reinterpret_cast<f32x4 *>(red + wave * (32 * TJ) + (x * 16 + a) * TJ + y * 16 + g * 4) = acc[x][y];
+    __syncthreads();
+
+    // wavefront tiles are added in wavefront order; 4 consecutive elements of the requested layout per thread
+    const bool eji = p.dw_layout != 0;
+    for (int item = tid; item < 8 * TJ; item += NW * 64) {
+        // EIJ: major = i (32 of them), TJ / 4 groups of four j;  EJI: major = j (TJ of them), 8 groups of four i
+        const int major = eji ? item >> 3 : item / (TJ / 4);
+        const int minor4 = (eji ? item & 7 : item % (TJ / 4)) * 4;
+        f32x4 v;
+        if (!eji) {
+            v = *reinterpret_cast<const f32x4 *>(red + major * TJ + minor4);
+#pragma unroll
+            for (int w = 1; w < NW; ++w) {
+                const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * (32 * TJ) + major * TJ + minor4);
+                v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+            }
+        } else {
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                float s1 = red[(minor4 + x) * TJ + major];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) s1 += red[w * (32 * TJ) + (minor4 + x) * TJ + major];
+                v[x] = s1;
+            }
+        }
+        const int gi = i0 + (eji ? minor4 : major), gj = j0 + (eji ? major : minor4);
+        if (gi >= p.I || gj >= p.J) continue;           // I % 4 == 0 and J % 4 == 0: a group of 4 is inside or outside
+        const size_t at = eji ? ((size_t)e * p.J + gj) * p.I + gi : ((size_t)e * p.I + gi) * p.J + gj;
+        if (p.out_dtype == 0) {
+            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.dW) + at) = v;
+        } else {
+            u32x2 w2;
+            w2[0] = p.out_dtype == 1 ? pack2<ElemF16>(v[0], v[1]) : pack2<ElemBF16>(v[0], v[1]);
+            w2[1] = p.out_dtype == 1 ? pack2<ElemF16>(v[2], v[3]) : pack2<ElemBF16>(v[2], v[3]);
+            *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.dW) + at) = w2;
+        }
+    }
+}
+
+template <class TT>
+__global__ __launch_bounds__(kThreads) void dw_tile_kernel(DwTileParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_dw_tile[];
+    dw_tile_body<TT, kThreads / 64>(p, (int)blockIdx.x, smem_dw_tile);
+}
+
+// 32 x 64 tiles, 8 wavefronts
+constexpr int kDwWideThreads = 512;
+template <class TT>
+__global__ __launch_bounds__(kDwWideThreads) void dw_tile_wide_kernel(DwTileParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_dw_tile_wide[];
+    dw_tile_body<TT, kDwWideThreads / 64, 64>(p, (int)blockIdx.x, smem_dw_tile_wide);
+}
+
+}  // namespace egs

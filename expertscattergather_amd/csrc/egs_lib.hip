@@ -6,6 +6,7 @@
 #include "egs_device.h"
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
+#include "egs_dw_tile.h"
 #include "egs_scatter_fused.h"
 
 #include <atomic>
@@ -217,6 +218,14 @@ struct SmallDwJob {
     bool done;          // set once the first pass has been enqueued
 };
 
+// one launch of dw_tile_kernel (or its share of a heterogeneous launch): the whole weight gradient, no second pass
+struct DwTileJob {
+    DwTileParams q;
+    int blocks, act_dtype;
+    bool wide;          // 32 x 64 tiles and 8 wavefronts (dw_tile_wide_kernel) instead of 32 x 32 and 4
+    bool done;          // set once it has been enqueued
+};
+
 bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
                        int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, SmallRowsJob &j)
 {
@@ -300,10 +309,90 @@ bool make_dw_small(const void *Xs, const void *Ys, const void *Ind, void *dW, vo
     return true;
 }
 
-// ---- launch of a rows job, alone or sharing the launch with the first pass of a dW job
-template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
-int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+// The one-pass weight gradient (32 x 32 tiles of dW(e), every workgroup reduces all picks of its expert) is taken
+// when its tiles alone fill the device; with fewer tiles the picks are split instead (dw_small_kernel + second pass).
+bool make_dw_tile(const void *Xs, const void *Ys, const void *Ind, void *dW, const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                  int act_dtype, int out_dtype, int ind_dtype, int dw_layout, DwTileJob &j, bool wide = false)
 {
+    if (g_force_generic || act_dtype == EGS_F32) return false;
+    if (d->I % 8 || d->J % 8 || d->I < 8 || d->J < 8 || d->I > 128 || d->J > 128) return false;
+    const int64_t Me = (int64_t)d->B * d->K;
+    if (Me == 0 || d->E == 0 || d->T == 0) return false;
+    const int it = ceil_div(d->I, 32), jt = ceil_div(d->J, wide ? 64 : 32);
+    if ((int64_t)d->E * it * jt < (wide ? 64 : 128)) return false;
+    if (!aligned_to(Xs, 16) || !aligned_to(Ys, 16) || !aligned_to(dW, 16) || (ldx_b * 2) % 16 || (ldx_t * 2) % 16) return false;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * 2;
+    const uint64_t y_span = (uint64_t)Me * d->E * d->J * 2;
+    if (x_span >= (1ull << 31) || y_span >= (1ull << 31)) return false;
+    if ((int64_t)8 * ceil_div(d->E, 8) * it * jt > INT32_MAX / 2) return false;
+    memset(&j, 0, sizeof(j));
+    DwTileParams &q = j.q;
+    q.Xs = (const char *)Xs; q.Ys = (const char *)Ys; q.Ind = Ind; q.dW = (char *)dW;
+    q.B = d->B; q.T = d->T; q.E = d->E; q.K = d->K; q.I = d->I; q.J = d->J;
+    q.ldx_b = ldx_b; q.ldx_t = ldx_t; q.ind_dtype = ind_dtype;
+    q.i_tiles = it; q.j_tiles = jt;
+    q.out_dtype = out_dtype; q.dw_layout = dw_layout;
+    q.x_bytes = (uint32_t)x_span; q.y_bytes = (uint32_t)y_span;
+    j.blocks = 8 * ceil_div(d->E, 8) * it * jt;
+    j.act_dtype = act_dtype;
+    j.wide = wide;
+    return true;
+}
+
+int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
+{
+    if (j.wide) {
+        static LdsGrant told_bf16, told_f16;
+        const size_t lds = dw_tile_lds(kDwWideThreads / 64, 64);
+        const int rc = j.act_dtype == EGS_BF16
+            ? allow_large_lds((const void *)dw_tile_wide_kernel<ElemBF16>, told_bf16, lds, "hipFuncSetAttribute(dw_tile_wide_kernel)")
+            : allow_large_lds((const void *)dw_tile_wide_kernel<ElemF16>, told_f16, lds, "hipFuncSetAttribute(dw_tile_wide_kernel)");
+        if (rc != EGS_OK) return rc;
+        if (j.act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_tile_wide_kernel<ElemBF16>, dim3(j.blocks), dim3(kDwWideThreads), lds, s, j.q);
+        else hipLaunchKernelGGL(dw_tile_wide_kernel<ElemF16>, dim3(j.blocks), dim3(kDwWideThreads), lds, s, j.q);
+    } else {
+        const size_t lds = dw_tile_lds(kThreads / 64);
+        if (j.act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_tile_kernel<ElemBF16>, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
+        else hipLaunchKernelGGL(dw_tile_kernel<ElemF16>, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
+    }
+    EGS_CHECK_LAUNCH("dw_tile_kernel");
+    j.done = true;
+    return EGS_OK;
+}
+
+// number of CUs of the current device (looked up once per device)
+int device_cu_count()
+{
+    static std::atomic<int> cached[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
+// ---- launch of a rows job, alone or sharing the launch with a weight gradient of the same call (its one-pass form,
+// or the first pass of its split form)
+template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
+int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
+{
+    if constexpr (GATHER) {
+        if (dwt != nullptr) {       // dwt->wide, and j regridded for 8 wavefronts per workgroup (see pair_gather_with_dw_tile)
+            static LdsGrant told;
+            const size_t tile_lds = dw_tile_lds(kDwWideThreads / 64, 64);
+            const int rc = allow_large_lds((const void *)rows_dw_tile_kernel<TT, W_NMAJOR, KS, TN>, told, tile_lds,
+                                           "hipFuncSetAttribute(rows_dw_tile_kernel)");
+            if (rc != EGS_OK) return rc;
+            hipLaunchKernelGGL((rows_dw_tile_kernel<TT, W_NMAJOR, KS, TN>), dim3(j.blocks + dwt->blocks), dim3(kDwWideThreads),
+                               tile_lds, s, j.p, dwt->q, j.blocks);
+            EGS_CHECK_LAUNCH("rows_dw_tile_kernel");
+            dwt->done = true;
+            return EGS_OK;
+        }
+    }
     if (dw != nullptr) {
         hipLaunchKernelGGL((rows_dw_small_kernel<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>), dim3(j.blocks + dw->blocks),
                            dim3(kThreads), j.lds, s, j.p, dw->q, j.blocks);
@@ -317,35 +406,36 @@ int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
 }
 
 template <class TT, bool W_NMAJOR, int TN, bool GATHER, bool OUT_F32>
-int launch_rows_small_ks(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+int launch_rows_small_ks(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
     switch (j.R) {
-    case 32: return launch_rows_small_one<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>(j, dw, s);
-    case 64: return launch_rows_small_one<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>(j, dw, s);
-    default: return launch_rows_small_one<TT, W_NMAJOR, 4, TN, GATHER, OUT_F32>(j, dw, s);
+    case 32: return launch_rows_small_one<TT, W_NMAJOR, 1, TN, GATHER, OUT_F32>(j, dw, dwt, s);
+    case 64: return launch_rows_small_one<TT, W_NMAJOR, 2, TN, GATHER, OUT_F32>(j, dw, dwt, s);
+    default: return launch_rows_small_one<TT, W_NMAJOR, 4, TN, GATHER, OUT_F32>(j, dw, dwt, s);
     }
 }
 
 template <class TT, bool GATHER, bool OUT_F32>
-int launch_rows_small_tn(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+int launch_rows_small_tn(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
     if (j.p.N <= 64)
-        return j.nmajor ? launch_rows_small_ks<TT, true, 4, GATHER, OUT_F32>(j, dw, s)
-                        : launch_rows_small_ks<TT, false, 4, GATHER, OUT_F32>(j, dw, s);
-    return j.nmajor ? launch_rows_small_ks<TT, true, 8, GATHER, OUT_F32>(j, dw, s)
-                    : launch_rows_small_ks<TT, false, 8, GATHER, OUT_F32>(j, dw, s);
+        return j.nmajor ? launch_rows_small_ks<TT, true, 4, GATHER, OUT_F32>(j, dw, dwt, s)
+                        : launch_rows_small_ks<TT, false, 4, GATHER, OUT_F32>(j, dw, dwt, s);
+    return j.nmajor ? launch_rows_small_ks<TT, true, 8, GATHER, OUT_F32>(j, dw, dwt, s)
+                    : launch_rows_small_ks<TT, false, 8, GATHER, OUT_F32>(j, dw, dwt, s);
 }
 
 template <class TT>
-int launch_rows_small_tt(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+int launch_rows_small_tt(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
-    if (j.gather) return launch_rows_small_tn<TT, true, false>(j, dw, s);
-    return j.out_f32 ? launch_rows_small_tn<TT, false, true>(j, dw, s) : launch_rows_small_tn<TT, false, false>(j, dw, s);
+    if (j.gather) return launch_rows_small_tn<TT, true, false>(j, dw, dwt, s);
+    return j.out_f32 ? launch_rows_small_tn<TT, false, true>(j, dw, dwt, s) : launch_rows_small_tn<TT, false, false>(j, dw, dwt, s);
 }
 
-int launch_rows_small_job(SmallRowsJob &j, SmallDwJob *dw, hipStream_t s)
+// `dwt` (one-pass weight gradient) shares the launch of a gather only; `dw` (first pass of the split form) any rows job
+int launch_rows_small_job(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
-    return j.act_dtype == EGS_BF16 ? launch_rows_small_tt<ElemBF16>(j, dw, s) : launch_rows_small_tt<ElemF16>(j, dw, s);
+    return j.act_dtype == EGS_BF16 ? launch_rows_small_tt<ElemBF16>(j, dw, dwt, s) : launch_rows_small_tt<ElemF16>(j, dw, dwt, s);
 }
 
 int launch_dw_small_alone(SmallDwJob &j, hipStream_t s)
@@ -451,11 +541,22 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
 
 // ------------------------------------------------------------------------------ fused small-expert scatter
 template <class TT, bool W_NMAJOR, int KS>
-int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
+int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
-    static LdsGrant told_plain, told_dw;        // one pair per template instantiation
-    if constexpr (TT::ES != 2) dw = nullptr;            // the small weight gradient exists for 16-bit types only
-    if (dw != nullptr) {
+    static LdsGrant told_plain, told_dw, told_dwt;      // one set per template instantiation
+    if constexpr (TT::ES != 2) { dw = nullptr; dwt = nullptr; }     // the small weight gradients exist for 16-bit types only
+    if (dwt != nullptr) {
+      if constexpr (TT::ES == 2) {
+        const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
+        const size_t need = lds > tile_lds ? lds : tile_lds;
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_dwtile_kernel<TT, W_NMAJOR, KS>, told_dwt, need,
+                                           "hipFuncSetAttribute(scatter_fused_dwtile_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
+        hipLaunchKernelGGL((scatter_fused_dwtile_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dwt->blocks), dim3(kFusedThreads), need,
+                           s, p, dwt->q, blocks);
+        dwt->done = true;
+      }
+    } else if (dw != nullptr) {
       if constexpr (TT::ES == 2) {
         const size_t dw_lds = (size_t)kDwSmallLdsBytes * (kFusedThreads / kThreads);       // one 16 KB tile per wavefront
         const size_t need = lds > dw_lds ? lds : dw_lds;
@@ -477,19 +578,19 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
 }
 
 template <class TT, bool W_NMAJOR>
-int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int blocks, SmallDwJob *dw, hipStream_t s)
+int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int blocks, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
     switch (R / (4 * TT::VEC)) {        // MFMA steps of four 16-byte chunks
-    case 1: return launch_scatter_fused_one<TT, W_NMAJOR, 1>(p, lds, blocks, dw, s);
-    case 2: return launch_scatter_fused_one<TT, W_NMAJOR, 2>(p, lds, blocks, dw, s);
-    default: return launch_scatter_fused_one<TT, W_NMAJOR, 4>(p, lds, blocks, dw, s);
+    case 1: return launch_scatter_fused_one<TT, W_NMAJOR, 1>(p, lds, blocks, dw, dwt, s);
+    case 2: return launch_scatter_fused_one<TT, W_NMAJOR, 2>(p, lds, blocks, dw, dwt, s);
+    default: return launch_scatter_fused_one<TT, W_NMAJOR, 4>(p, lds, blocks, dw, dwt, s);
     }
 }
 
 // GEMM-scatter of small experts in one kernel (product rows stay in LDS); `used` reports whether the
 // shape qualified.  Both scatter modes take it: it is bitwise reproducible and needs no workspace.
 int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
-                  int w_layout, SmallDwJob *dw, hipStream_t s, bool &used)
+                  int w_layout, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s, bool &used)
 {
     used = false;
     const int R = d->J, N = d->I;
@@ -515,13 +616,13 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     used = true;
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
     if (act_dtype == EGS_F32)
-        return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, s)
-                      : launch_scatter_fused_ks<ElemF32, false>(p, R, lds, (int)blocks, nullptr, s);
+        return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, nullptr, s)
+                      : launch_scatter_fused_ks<ElemF32, false>(p, R, lds, (int)blocks, nullptr, nullptr, s);
     if (act_dtype == EGS_F16)
-        return nmajor ? launch_scatter_fused_ks<ElemF16, true>(p, R, lds, (int)blocks, dw, s)
-                      : launch_scatter_fused_ks<ElemF16, false>(p, R, lds, (int)blocks, dw, s);
-    return nmajor ? launch_scatter_fused_ks<ElemBF16, true>(p, R, lds, (int)blocks, dw, s)
-                  : launch_scatter_fused_ks<ElemBF16, false>(p, R, lds, (int)blocks, dw, s);
+        return nmajor ? launch_scatter_fused_ks<ElemF16, true>(p, R, lds, (int)blocks, dw, dwt, s)
+                      : launch_scatter_fused_ks<ElemF16, false>(p, R, lds, (int)blocks, dw, dwt, s);
+    return nmajor ? launch_scatter_fused_ks<ElemBF16, true>(p, R, lds, (int)blocks, dw, dwt, s)
+                  : launch_scatter_fused_ks<ElemBF16, false>(p, R, lds, (int)blocks, dw, dwt, s);
 }
 
 // ------------------------------------------------------------------------------ implementations
@@ -533,7 +634,7 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
     if (w_scale == nullptr) {
         SmallRowsJob j;
         if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j))
-            return launch_rows_small_job(j, nullptr, s);
+            return launch_rows_small_job(j, nullptr, nullptr, s);
     }
     RowsGemmParams p;
     memset(&p, 0, sizeof(p));
@@ -559,7 +660,7 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
 // launch and whose second pass may share the reduction launch
 int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, void *workspace,
                       const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode, SmallDwJob *dw,
-                      hipStream_t s)
+                      DwTileJob *dwt, hipStream_t s)
 {
     const int ES = elem_size(act_dtype);
     const size_t out_elems = (size_t)d->B * d->T * d->I;
@@ -595,7 +696,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
 
     {   // small experts: everything in one kernel
         bool used = false;
-        const int rc_fused = scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, s, used);
+        const int rc_fused = scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s, used);
         if (used) return rc_fused;
     }
 
@@ -619,7 +720,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
             rc = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, long_tab, s);
             if (rc != EGS_OK) return rc;
         }
-        rc = launch_rows_small_job(j, dw, s);
+        rc = launch_rows_small_job(j, dw, nullptr, s);
     } else {
         rows_f32 = mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32;   // fast mode: rows in the element type
         // Product rows that one launch writes and the next reads back are still in the 256 MB memory-side
@@ -677,6 +778,9 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
 {
     if ((size_t)d->E * d->I * d->J == 0) return EGS_OK;
     const DwPlan pl = plan_dw(d, act_dtype);
+    DwTileJob jt;
+    if (make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt))
+        return launch_dw_tile_alone(jt, s);
     SmallDwJob j;
     if (make_dw_small(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, j)) {
         int rc = launch_dw_small_alone(j, s);
@@ -817,7 +921,8 @@ int egs_gemm_scatter(const void *Y, const void *W, const void *Ind, void *Out,
 {
     int rc = validate_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, act_dtype, ind_dtype, w_layout, mode);
     if (rc != EGS_OK) return rc;
-    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, act_dtype, ind_dtype, w_layout, mode, nullptr, (hipStream_t)stream);
+    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, act_dtype, ind_dtype, w_layout, mode, nullptr, nullptr,
+                             (hipStream_t)stream);
 }
 
 int egs_dw(const void *Xsrc, const void *Ysrc, const void *Ind, void *dW,
@@ -889,11 +994,15 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     const size_t w_elems = (size_t)d->E * d->I * d->J;
     const DwPlan dpl = plan_dw(d, dtype);
     SmallDwJob dwj;
-    const bool dw_small = w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype,
-                                                       EGS_W_EIJ, dpl, dwj);
-    rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr, s);
+    DwTileJob dwt;
+    const bool dw_tile = w_elems > 0 && make_dw_tile(X, grad_Y, Ind, grad_W, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dwt);
+    const bool dw_small = !dw_tile && w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype,
+                                                                   ind_dtype, EGS_W_EIJ, dpl, dwj);
+    rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr,
+                           dw_tile ? &dwt : nullptr, s);
     if (rc != EGS_OK) return rc;
     if (w_elems == 0) return EGS_OK;
+    if (dw_tile) return dwt.done ? EGS_OK : launch_dw_tile_alone(dwt, s);
     if (dw_small) {
         if (!dwj.done) { rc = launch_dw_small_alone(dwj, s); if (rc != EGS_OK) return rc; }
         return launch_dw_reduce4(dwj, s);       // no-op when the reduction launch already did it
@@ -928,10 +1037,30 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
     SmallDwJob dwj;
     const bool g_small = y_elems > 0 && make_gather_small(grad_Out, W, Ind, grad_Y, d, ldg_b, ldg_t, dtype, dtype, ind_dtype,
                                                           EGS_W_EJI, gj);
-    const bool dw_small = w_elems > 0 && make_dw_small(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype,
-                                                       ind_dtype, EGS_W_EJI, dpl, dwj);
+    DwTileJob dwt;
+    if (g_small && w_elems > 0 &&
+        make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt, /*wide=*/true)) {
+        // one launch, every workgroup on a CU of its own: the gather regridded to 8 wavefronts per workgroup
+        SmallRowsJob g8 = gj;
+        const int64_t Me = (int64_t)d->B * d->K;
+        g8.p.tiles_per_e = (int)((Me + 511) / 512);
+        if (g8.p.tiles_per_e % 8 != 0) g8.p.rows_share_xcd = 0;     // row tiles map to XCDs in groups of 8 only
+        g8.blocks = g8.p.rows_share_xcd ? 8 * ceil_div(g8.p.tiles_per_e, 8) * g8.p.E : 8 * ceil_div(g8.p.E, 8) * g8.p.tiles_per_e;
+        const int cus = device_cu_count();
+        if (cus > 0 && g8.blocks + dwt.blocks <= cus) return launch_rows_small_job(g8, nullptr, &dwt, s);
+    }
+    const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt);
+    if (dw_tile) {
+        if (y_elems > 0) {
+            rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);
+            if (rc != EGS_OK) return rc;
+        }
+        return launch_dw_tile_alone(dwt, s);
+    }
+    const bool dw_small = !dw_tile && w_elems > 0 && make_dw_small(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype,
+                                                                   dtype, ind_dtype, EGS_W_EJI, dpl, dwj);
     if (g_small && dw_small) {
-        rc = launch_rows_small_job(gj, &dwj, s);
+        rc = launch_rows_small_job(gj, &dwj, nullptr, s);
         if (rc != EGS_OK) return rc;
         return launch_dw_reduce4(dwj, s);
     }

@@ -235,4 +235,16 @@ __global__ __launch_bounds__(kFusedThreads) void scatter_fused_dw_kernel(Scatter
     }
 }
 
+// ... or with the one-pass weight gradient (egs_dw_tile.h) of the same backward call
+template <class TT, bool W_NMAJOR, int KS>
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_dwtile_kernel(ScatterFusedParams p, DwTileParams q, int fused_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_fused_dwtile[];
+    if ((int)blockIdx.x < fused_blocks) {
+        scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused_dwtile);
+    } else {
+        if constexpr (TT::ES == 2) dw_tile_body<TT, kFusedThreads / 64>(q, (int)blockIdx.x - fused_blocks, smem_fused_dwtile);
+    }
+}
+
 }  // namespace egs

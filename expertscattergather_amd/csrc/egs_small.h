@@ -25,6 +25,7 @@
 #pragma once
 #include "egs_device.h"
 #include "egs_scatter_aux.h"
+#include "egs_dw_tile.h"
 
 namespace egs {
 
@@ -45,7 +46,8 @@ struct SmallRowsParams {
 
 // Requirements (checked by the launcher): 2-byte elements, R == 32*KS, N % 8 == 0,
 // 8 <= N <= 16*TN, A rows / W / C 16-byte aligned, every tensor smaller than 4 GiB.
-template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
+// WPB = wavefronts per workgroup (a workgroup covers 64 * WPB picks of one expert; tiles_per_e counts such workgroups)
+template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32, int WPB = 4>
 __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const int block, int32_t *sh_cnt_small)
 {
     constexpr int TQ = 4;                       // 4 row tiles = 64 picks per wave
@@ -54,7 +56,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     static_assert(!(GATHER && OUT_F32), "gather results are stored in the element type");
     if constexpr (!GATHER) {
         if (block < p.csr_blocks) {
-            csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, kThreads, p.Ind, p.ind_dtype, p.T,
+            csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
                            p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
             return;
         }
@@ -66,7 +68,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: scalar address work
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
-    const int m0 = (tile * 4 + wave) * 64;
+    const int m0 = (tile * WPB + wave) * 64;
     if (m0 >= Me) return;                       // no barriers below: a wave may leave alone
     const int N = p.N;
 
@@ -468,6 +470,22 @@ __global__ __launch_bounds__(kThreads) void rows_dw_small_kernel(SmallRowsParams
     __shared__ __attribute__((aligned(16))) float red[kDwSmallLdsBytes / 4];
     if ((int)blockIdx.x < rows_blocks) rows_small_body<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>(p, (int)blockIdx.x, sh_dyn_fused);
     else dw_small_body<TT>(q, (int)blockIdx.x - rows_blocks, red);
+}
+
+// A gather and the one-pass weight gradient (egs_dw_tile.h, 32 x 64 tiles) of the same backward call in one launch.
+// Both kinds of workgroup have 8 wavefronts and the kernel's register and LDS footprint admits one workgroup per
+// CU: when the launcher chooses this kernel the two kinds together have no more workgroups than the device has
+// CUs, so every workgroup gets a CU of its own and the two kinds do not compete for a CU's path to the L2 (which
+// is what bounds the weight gradient; sharing CUs made the pair as slow as running one after the other).
+template <class TT, bool W_NMAJOR, int KS, int TN>
+__global__ __launch_bounds__(kDwWideThreads) void rows_dw_tile_kernel(SmallRowsParams p, DwTileParams q, int rows_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) char sh_dyn_rows_tile[];
+    // the weight gradient's workgroups (the longer ones) come first in launch order
+    const int dw_blocks = (int)gridDim.x - rows_blocks;
+    if ((int)blockIdx.x < dw_blocks) dw_tile_body<TT, kDwWideThreads / 64, 64>(q, (int)blockIdx.x, sh_dyn_rows_tile);
+    else rows_small_body<TT, W_NMAJOR, KS, TN, true, false, kDwWideThreads / 64>(p, (int)blockIdx.x - dw_blocks,
+                                                                                  reinterpret_cast<int32_t *>(sh_dyn_rows_tile));
 }
 
 // segment sums of a scatter and the second pass of a weight gradient in one launch:
