@@ -26,6 +26,7 @@ from . import _abi
 __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
     "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
+    "register_reference_namespace", "release_workspaces",
 ]
 
 OP_NAMESPACE = "egs_amd"
@@ -113,27 +114,23 @@ def _on_device(dev: torch.device):
     return torch.cuda.device(dev)
 
 
-_workspaces: dict = {}
-
-
 def _workspace(dev: torch.device, nbytes: int):
-    """Scratch buffer per (device, stream), grown on demand; returns (ptr, nbytes)."""
+    """Scratch for one call: (tensor that owns it or None, pointer, nbytes).
+
+    Allocated per call through torch's caching allocator, which is stream-ordered and aware of graph
+    capture: a buffer handed out during capture belongs to the graph's pool and stays valid for every
+    replay, and a buffer of an eager call is not reused by another stream before the call's kernels have
+    run.  (A buffer cached across calls would have its address baked into captured graphs and could be
+    freed or regrown underneath them.)  The caller keeps the tensor alive until the launch is enqueued."""
     if nbytes == 0:
-        return None, 0
-    key = (dev.index, _stream_ptr(dev))
-    buf = _workspaces.get(key)
-    if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(int(nbytes * 1.25) + 256, dtype=torch.uint8, device=dev)
-        _workspaces[key] = buf
-    return buf.data_ptr(), buf.numel()
+        return None, None, 0
+    buf = torch.empty(int(nbytes), dtype=torch.uint8, device=dev)
+    return buf, buf.data_ptr(), int(nbytes)
 
 
 def release_workspaces() -> None:
-    """Drop the cached scratch buffers (one per device and stream that has run a scatter or a backward).
-
-    They are re-created on demand; call this after a burst of work on short-lived streams, or
-    before measuring peak memory."""
-    _workspaces.clear()
+    """Kept for callers of earlier versions, which cached one scratch buffer per stream; scratch is now
+    allocated per call, so there is nothing to release."""
 
 
 def _rows_source(X: torch.Tensor):
@@ -167,90 +164,107 @@ def _check_shapes(X3, W, Ind, Y4, w_is_eij: bool):
     return B, E, K, I, J
 
 
-def _same_dtype(*tensors):
-    dt = tensors[0].dtype
-    for t in tensors[1:]:
-        if t.dtype != dt:
-            raise ValueError(f"activations and weights must share one dtype, got {dt} and {t.dtype}")
-    return dtype_to_type_id(dt)
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def _compute_dtype(out_dtype: torch.dtype, *tensors: torch.Tensor) -> torch.dtype:
+    """The element type the kernels multiply in, following the reference's kernels (egs/triton_kernels.py:122-127,
+    :131-136): ``out_dtype`` float16 / bfloat16 casts both operands to it; float32 leaves them as they are, i.e.
+    operands that already share a 16-bit type are multiplied in that type (fp32 accumulation either way), and
+    operands of different types meet in float32.  Results are returned in the dtype of the tensor they are the
+    gradient of / the activation they continue (:375, :408-409, :457, :491-492)."""
+    dtype_to_type_id(out_dtype)
+    for t in tensors:
+        if t.dtype not in _FLOATS:
+            raise ValueError("Unknown dtype")
+    if out_dtype != torch.float32:
+        return out_dtype
+    first = tensors[0].dtype
+    return first if all(t.dtype == first for t in tensors) else torch.float32
 
 
 # ------------------------------------------------------------------------------ the four launchers
 def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    dtype_to_type_id(out_dtype)
+    ct = _compute_dtype(out_dtype, X, W)
     dev = _require_gpu(X, W, Ind)
     B, E, K, I, J = _check_shapes(X, W, Ind, None, True)
-    dt = _same_dtype(X, W)
-    X, ld_b, ld_t = _rows_source(X)
-    W = W.contiguous(); Ind = Ind.contiguous()
-    Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
+    res_dtype = X.dtype
+    X, ld_b, ld_t = _rows_source(X.to(ct))
+    W = W.to(ct).contiguous(); Ind = Ind.contiguous()
+    Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
     with _on_device(dev):
         rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
-                                                  ld_b, ld_t, dt, _ind_type_id(Ind), _stream_ptr(dev))
+                                                  ld_b, ld_t, dtype_to_type_id(ct), _ind_type_id(Ind), _stream_ptr(dev))
     _abi.check(rc, "expert_gather_forward_call")
-    return Y
+    return Y.to(res_dtype)
 
 
 def _gather_backward_impl(X, W, Ind, grad_output, dtype):
-    dtype_to_type_id(dtype)
+    ct = _compute_dtype(dtype, X, W, grad_output)
     dev = _require_gpu(X, W, Ind, grad_output)
     B, E, K, I, J = _check_shapes(X, W, Ind, grad_output, True)
-    dt = _same_dtype(X, W, grad_output)
-    X, ld_b, ld_t = _rows_source(X)
-    W = W.contiguous(); Ind = Ind.contiguous(); grad_output = grad_output.contiguous()
+    x_dtype, w_dtype = X.dtype, W.dtype
+    X, ld_b, ld_t = _rows_source(X.to(ct))
+    W = W.to(ct).contiguous(); Ind = Ind.contiguous(); grad_output = grad_output.to(ct).contiguous()
     T = X.shape[1]
-    grad_X = torch.empty((B, T, I), device=dev, dtype=X.dtype)
-    grad_W = torch.empty((E, I, J), device=dev, dtype=W.dtype)
+    grad_X = torch.empty((B, T, I), device=dev, dtype=ct)
+    grad_W = torch.empty((E, I, J), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
+    dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt))
         rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
                                                    grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                    dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+    del keep
     _abi.check(rc, "expert_gather_backward_call")
-    return grad_X, grad_W
+    return grad_X.to(x_dtype), grad_W.to(w_dtype)
 
 
 def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
-    dtype_to_type_id(out_dtype)
+    ct = _compute_dtype(out_dtype, Y, W)
     dev = _require_gpu(Y, W, Ind)
     B, E, K, I, J = _check_shapes(None, W, Ind, Y, False)
-    dt = _same_dtype(Y, W)
     T = int(T)
     if T < 0:
         raise ValueError("T must be non-negative")
-    Y = Y.contiguous(); W = W.contiguous(); Ind = Ind.contiguous()
-    out = torch.empty((B, T, I), device=dev, dtype=Y.dtype)
+    res_dtype = Y.dtype
+    Y = Y.to(ct).contiguous(); W = W.to(ct).contiguous(); Ind = Ind.contiguous()
+    out = torch.empty((B, T, I), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
+    dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt))
         rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
                                                    ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+    del keep
     _abi.check(rc, "expert_scatter_forward_call")
-    return out
+    return out.to(res_dtype)
 
 
 def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
-    dtype_to_type_id(dtype)
+    ct = _compute_dtype(dtype, Y, W, grad_X)
     dev = _require_gpu(Y, W, Ind, grad_X)
     B, E, K, I, J = _check_shapes(grad_X, W, Ind, Y, False)
-    dt = _same_dtype(Y, W, grad_X)
-    grad_X, ld_b, ld_t = _rows_source(grad_X)
-    Y = Y.contiguous(); W = W.contiguous(); Ind = Ind.contiguous()
+    y_dtype, w_dtype = Y.dtype, W.dtype
+    grad_X, ld_b, ld_t = _rows_source(grad_X.to(ct))
+    Y = Y.to(ct).contiguous(); W = W.to(ct).contiguous(); Ind = Ind.contiguous()
     T = grad_X.shape[1]
-    grad_Y = torch.empty((B, E, K, J), device=dev, dtype=Y.dtype)
-    grad_W = torch.empty((E, J, I), device=dev, dtype=W.dtype)
+    grad_Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
+    grad_W = torch.empty((E, J, I), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
+    dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, d, dt))
         rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
                                                     grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                     dt, _ind_type_id(Ind), _stream_ptr(dev))
+    del keep
     _abi.check(rc, "expert_scatter_backward_call")
-    return grad_Y, grad_W
+    return grad_Y.to(y_dtype), grad_W.to(w_dtype)
 
 
 # module globals, bound by create_kernels() (reference egs/triton_kernels.py:26-29)
@@ -259,6 +273,70 @@ expert_gather_backward_call = None
 expert_scatter_forward_call = None
 expert_scatter_backward_call = None
 _create_lock = threading.Lock()
+
+
+_libraries: dict = {}
+
+
+def _register_ops(ns: str) -> None:
+    """Define the four ops in namespace `ns` (schemas of reference egs/triton_kernels.py:362, :395, :444, :478), with
+    fake implementations for tracing and autograd formulas, so that the ops can also be called directly on tensors
+    that require grad and traced by torch.compile."""
+    lib = torch.library.Library(ns, "DEF")
+    lib.define("expert_gather_forward_call_fn(Tensor X, Tensor W, Tensor Ind, ScalarType out_dtype) -> Tensor")
+    lib.define("expert_gather_backward_call_fn(Tensor X, Tensor W, Tensor Ind, Tensor grad_output, "
+               "ScalarType out_dtype) -> (Tensor, Tensor)")
+    lib.define("expert_scatter_forward_call_fn(Tensor Y, Tensor W, Tensor Ind, int T, ScalarType out_dtype) -> Tensor")
+    lib.define("expert_scatter_backward_call_fn(Tensor Y, Tensor W, Tensor Ind, Tensor grad_X, "
+               "ScalarType out_dtype) -> (Tensor, Tensor)")
+    lib.impl("expert_gather_forward_call_fn", _gather_forward_impl, "CompositeExplicitAutograd")
+    lib.impl("expert_gather_backward_call_fn", _gather_backward_impl, "CompositeExplicitAutograd")
+    lib.impl("expert_scatter_forward_call_fn", _scatter_forward_impl, "CompositeExplicitAutograd")
+    lib.impl("expert_scatter_backward_call_fn", _scatter_backward_impl, "CompositeExplicitAutograd")
+
+    @torch.library.register_fake(f"{ns}::expert_gather_forward_call_fn", lib=lib)
+    def _(X, W, Ind, out_dtype):
+        return X.new_empty((X.shape[0], W.shape[0], Ind.shape[2], W.shape[2]))
+
+    @torch.library.register_fake(f"{ns}::expert_gather_backward_call_fn", lib=lib)
+    def _(X, W, Ind, grad_output, out_dtype):
+        return torch.empty_like(X, memory_format=torch.contiguous_format), torch.empty_like(
+            W, memory_format=torch.contiguous_format)
+
+    @torch.library.register_fake(f"{ns}::expert_scatter_forward_call_fn", lib=lib)
+    def _(Y, W, Ind, T, out_dtype):
+        return Y.new_empty((Y.shape[0], T, W.shape[2]))
+
+    @torch.library.register_fake(f"{ns}::expert_scatter_backward_call_fn", lib=lib)
+    def _(Y, W, Ind, grad_X, out_dtype):
+        return torch.empty_like(Y, memory_format=torch.contiguous_format), torch.empty_like(
+            W, memory_format=torch.contiguous_format)
+
+    ops = getattr(torch.ops, ns)
+
+    def gather_setup(ctx, inputs, output):
+        X, W, Ind, out_dtype = inputs
+        ctx.save_for_backward(X, W, Ind)
+        ctx.out_dtype = out_dtype
+
+    def gather_backward(ctx, grad_output):
+        X, W, Ind = ctx.saved_tensors
+        grad_X, grad_W = ops.expert_gather_backward_call_fn(X, W, Ind, grad_output, ctx.out_dtype)
+        return grad_X, grad_W, None, None
+
+    def scatter_setup(ctx, inputs, output):
+        Y, W, Ind, T, out_dtype = inputs
+        ctx.save_for_backward(Y, W, Ind)
+        ctx.out_dtype = out_dtype
+
+    def scatter_backward(ctx, grad_X):
+        Y, W, Ind = ctx.saved_tensors
+        grad_Y, grad_W = ops.expert_scatter_backward_call_fn(Y, W, Ind, grad_X, ctx.out_dtype)
+        return grad_Y, grad_W, None, None, None
+
+    torch.library.register_autograd(f"{ns}::expert_gather_forward_call_fn", gather_backward, setup_context=gather_setup, lib=lib)
+    torch.library.register_autograd(f"{ns}::expert_scatter_forward_call_fn", scatter_backward, setup_context=scatter_setup, lib=lib)
+    _libraries[ns] = lib            # keeps the registration alive
 
 
 def create_kernels() -> None:
@@ -274,43 +352,23 @@ def create_kernels() -> None:
     with _create_lock:
         if expert_scatter_backward_call is not None:
             return
-        ns = OP_NAMESPACE
-        lib = torch.library.Library(ns, "DEF")
-        lib.define("expert_gather_forward_call_fn(Tensor X, Tensor W, Tensor Ind, ScalarType out_dtype) -> Tensor")
-        lib.define("expert_gather_backward_call_fn(Tensor X, Tensor W, Tensor Ind, Tensor grad_output, "
-                   "ScalarType out_dtype) -> (Tensor, Tensor)")
-        lib.define("expert_scatter_forward_call_fn(Tensor Y, Tensor W, Tensor Ind, int T, ScalarType out_dtype) -> Tensor")
-        lib.define("expert_scatter_backward_call_fn(Tensor Y, Tensor W, Tensor Ind, Tensor grad_X, "
-                   "ScalarType out_dtype) -> (Tensor, Tensor)")
-        lib.impl("expert_gather_forward_call_fn", _gather_forward_impl, "CompositeExplicitAutograd")
-        lib.impl("expert_gather_backward_call_fn", _gather_backward_impl, "CompositeExplicitAutograd")
-        lib.impl("expert_scatter_forward_call_fn", _scatter_forward_impl, "CompositeExplicitAutograd")
-        lib.impl("expert_scatter_backward_call_fn", _scatter_backward_impl, "CompositeExplicitAutograd")
-
-        @torch.library.register_fake(f"{ns}::expert_gather_forward_call_fn", lib=lib)
-        def _(X, W, Ind, out_dtype):
-            return X.new_empty((X.shape[0], W.shape[0], Ind.shape[2], W.shape[2]))
-
-        @torch.library.register_fake(f"{ns}::expert_gather_backward_call_fn", lib=lib)
-        def _(X, W, Ind, grad_output, out_dtype):
-            return torch.empty_like(X, memory_format=torch.contiguous_format), torch.empty_like(
-                W, memory_format=torch.contiguous_format)
-
-        @torch.library.register_fake(f"{ns}::expert_scatter_forward_call_fn", lib=lib)
-        def _(Y, W, Ind, T, out_dtype):
-            return Y.new_empty((Y.shape[0], T, W.shape[2]))
-
-        @torch.library.register_fake(f"{ns}::expert_scatter_backward_call_fn", lib=lib)
-        def _(Y, W, Ind, grad_X, out_dtype):
-            return torch.empty_like(Y, memory_format=torch.contiguous_format), torch.empty_like(
-                W, memory_format=torch.contiguous_format)
-
-        create_kernels._lib = lib        # keep the registration alive
-        ops = getattr(torch.ops, ns)
+        _register_ops(OP_NAMESPACE)
+        ops = getattr(torch.ops, OP_NAMESPACE)
         expert_gather_forward_call = ops.expert_gather_forward_call_fn
         expert_gather_backward_call = ops.expert_gather_backward_call_fn
         expert_scatter_forward_call = ops.expert_scatter_forward_call_fn
         expert_scatter_backward_call = ops.expert_scatter_backward_call_fn
+
+
+def register_reference_namespace(ns: str = "mylib") -> None:
+    """Also expose the four ops as ``torch.ops.mylib.*``, the namespace the reference registers them under
+    (egs/triton_kernels.py:362), for code that addresses the ops by name instead of through the module-level
+    callables.  Optional and explicit because an op name can be defined only once per process: it raises if the
+    reference package (or anything else) has already defined these names."""
+    create_kernels()
+    with _create_lock:
+        if ns not in _libraries:
+            _register_ops(ns)
 
 
 # ------------------------------------------------------------------------------ autograd Functions
@@ -345,7 +403,9 @@ class ExpertScatterFunction(torch.autograd.Function):
     def backward(ctx, grad_X: torch.Tensor):
         Y, W, Ind = ctx.saved_tensors
         grad_Y, grad_W = expert_scatter_backward_call(Y, W, Ind, grad_X, ctx.dtype)
-        return grad_Y, grad_W, None, None
+        # one gradient per forward input: (Y, W, Ind, T) or (Y, W, Ind, T, out_type).  The reference returns four
+        # (egs/triton_kernels.py:639), which autograd rejects when out_type is passed explicitly.
+        return (grad_Y, grad_W) + (None,) * (len(ctx.needs_input_grad) - 2)
 
 
 # ------------------------------------------------------------------------------ extras (not in the reference)
@@ -391,11 +451,8 @@ def expert_gather_fp8_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.Te
     Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
     d = _abi.Dims(B, T, E, K, I, J)
     nbytes = _abi.lib().egs_gather_gemm_fp8act_workspace_bytes(d)
-    if return_quantised:
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
-        ws_ptr = ws.data_ptr()
-    else:
-        ws, (ws_ptr, _) = None, _workspace(dev, nbytes)
+    ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+    ws_ptr = ws.data_ptr()
     with _on_device(dev):
         rc = _abi.lib().egs_gather_gemm_fp8act(X.data_ptr(), Wq.data_ptr(), scale.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
                                                ws_ptr, nbytes, d, ld_b, ld_t, _ind_type_id(Ind), _stream_ptr(dev))

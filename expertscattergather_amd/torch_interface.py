@@ -71,13 +71,16 @@ class ExpertScatter(nn.Module):
     def forward(self, Y: torch.Tensor, Ind: torch.Tensor, T: int):
         """Y: [B,E,K,J];  Ind: [B,E,K] in [0,T);  T: output sequence length  ->  [B,T,I]."""
         y = ExpertScatterFunction.apply(Y, self.W, Ind, T)
-        if self.bias is not None:
+        if self.bias is not None and T > 0 and Ind.numel() > 0:
             # picks[b,t,e] = how many times expert e selected token t; each adds bias[e]
+            # (a pick outside [0,T) contributes nothing, as in the kernels: it is routed to slot 0 with weight 0)
             B, E, K = Ind.shape
             picks = torch.zeros(B, T, E, device=y.device, dtype=torch.float32)
             e_ids = torch.arange(E, device=y.device).view(1, E, 1).expand(B, E, K).reshape(B, E * K)
-            flat = Ind.to(torch.int64).reshape(B, E * K) * E + e_ids
-            picks.view(B, T * E).scatter_add_(1, flat, torch.ones_like(flat, dtype=torch.float32))
+            ind = Ind.to(torch.int64).reshape(B, E * K)
+            valid = (ind >= 0) & (ind < T)
+            flat = torch.where(valid, ind * E + e_ids, torch.zeros_like(ind))
+            picks.view(B, T * E).scatter_add_(1, flat, valid.to(torch.float32))
             y = y + (picks @ self.bias[:, 0, :].float()).to(y.dtype)
         return y
 

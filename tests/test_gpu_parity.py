@@ -220,8 +220,14 @@ def test_scatter_output_does_not_depend_on_stale_memory(mode):
 
 
 @pytest.mark.parametrize("shape,dtype", [((2, 20, 3, 6, 32, 16), torch.float32),
-                                         ((2, 300, 3, 260, 192, 256), torch.bfloat16)],     # second: 256 x 256 tile kernels
-                         ids=["small-f32", "large-bf16"])
+                                         ((2, 300, 3, 260, 192, 256), torch.bfloat16),      # 256 x 256 tile kernels
+                                         # small-expert kernels (register-resident gather, one-kernel scatter, split weight
+                                         # gradient); a rejected pick reads row 0 / a clamped address there and is masked
+                                         ((2, 64, 8, 16, 128, 64), torch.bfloat16),
+                                         # the same with enough experts for the one-pass weight gradient (its rejected picks
+                                         # get a buffer offset outside the descriptor) and its shared launch with the gather
+                                         ((8, 64, 32, 16, 128, 64), torch.float16)],
+                         ids=["small-f32", "large-bf16", "small-experts-bf16", "one-pass-dw-f16"])
 def test_out_of_range_picks_contribute_nothing(shape, dtype):
     B, T, E, K, I, J = shape
     case = make_case(13, B, T, E, K, I, J, dtype)
@@ -242,6 +248,9 @@ def test_out_of_range_picks_contribute_nothing(shape, dtype):
     dX, dWg = O.gather_backward(X, Wg, safe.numpy(), Y * mask)
     assert_close(got["dX"], dX, dtype, "dX with bad picks")
     assert_close(got["dWg"], dWg, dtype, "dWg with bad picks")
+    dYo, dWso = O.scatter_backward(Y * mask, Ws, safe.numpy(), dOut)
+    assert_close(got["dY"], dYo * mask, dtype, "dY with bad picks")
+    assert_close(got["dWs"], dWso, dtype, "dWs with bad picks")
 
 
 def test_strided_source_rows():
@@ -276,8 +285,8 @@ def test_errors_are_python_exceptions():
         hk.expert_gather_forward_call(X.double(), W.double(), Ind, torch.float32)
     with pytest.raises(ValueError, match="Unknown dtype"):
         hk.expert_gather_forward_call(X, W, Ind, torch.int32)
-    with pytest.raises(ValueError):
-        hk.expert_gather_forward_call(X, W.half(), Ind, torch.float32)
+    # mixed activation / weight dtypes are not an error (the reference casts inside its kernels): they meet in float32
+    assert hk.expert_gather_forward_call(X, W.half(), Ind, torch.float32).dtype == torch.float32
     with pytest.raises(ValueError):
         hk.expert_gather_forward_call(X, W, Ind.float(), torch.float32)
     with pytest.raises(RuntimeError, match="no CPU fallback"):
@@ -365,6 +374,18 @@ def test_gather_bias_and_scatter_bias():
             for k in range(K):
                 ref[b, int(case["Ind"][b, e, k])] += bias[e, 0]
     assert_close(out, ref, torch.float32, "scatter bias")
+    # a pick outside [0,T) adds neither its product row nor its expert's bias (and does not trip an index assert)
+    bad = case["Ind"].clone(); bad[0, 1, 2] = T + 5; bad[1, 0, 0] = -3
+    out2 = scatter(dev(case["Y"]), dev(bad), T)
+    live = ((bad >= 0) & (bad < T)).numpy()
+    safe = torch.where(torch.from_numpy(live), bad, torch.zeros_like(bad)).numpy()
+    ref2 = O.scatter_forward(np64(case["Y"]) * live[..., None], np64(scatter.W), safe, T)
+    for b in range(B):
+        for e in range(E):
+            for k in range(K):
+                if live[b, e, k]:
+                    ref2[b, int(bad[b, e, k])] += bias[e, 0]
+    assert_close(out2, ref2, torch.float32, "scatter bias with rejected picks")
 
 
 def test_fp8_weight_gather_matches_dequantised_oracle():
@@ -443,7 +464,7 @@ def test_ops_pass_opcheck_and_router_output_feeds_the_kernels():
     Ind, _ = expert_choice_router(dev(logits), K, torch.int32)
     X, Wg, Ws, Y, dOut = (dev(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut"))
     ops = torch.ops.egs_amd
-    tests = ("test_schema", "test_faketensor")
+    tests = ("test_schema", "test_faketensor", "test_autograd_registration", "test_aot_dispatch_dynamic")
     torch.library.opcheck(ops.expert_gather_forward_call_fn.default, (X, Wg, Ind, torch.float32), test_utils=tests)
     torch.library.opcheck(ops.expert_scatter_forward_call_fn.default, (Y, Ws, Ind, T, torch.float32), test_utils=tests)
     torch.library.opcheck(ops.expert_gather_backward_call_fn.default, (X, Wg, Ind, Y, torch.float32), test_utils=tests)
@@ -488,3 +509,67 @@ def test_graph_replays_match_eager_results(shape):
         for name, got, ref in zip(("Y", "out", "dX", "dWg", "dWs"), outs, eager):
             assert torch.equal(got, ref), f"replay {rep}: {name} differs from the eager result"
         del junk
+
+
+@pytest.mark.parametrize("out_type", [torch.bfloat16, torch.float32], ids=["out-bf16", "out-f32"])
+def test_mixed_precision_follows_the_reference_kernels(out_type):
+    """bf16 activations with fp32 parameters.  out_type bfloat16: the weights are rounded to bf16 and the products run in
+    bf16 (reference egs/triton_kernels.py:122-127); out_type float32: the operands meet in fp32.  Results come back in the
+    activation's dtype, weight gradients in the parameter's (:375, :408-409, :457, :491-492)."""
+    B, T, E, K, I, J = 3, 40, 6, 9, 64, 32
+    case = make_case(61, B, T, E, K, I, J, torch.bfloat16)
+    g = torch.Generator().manual_seed(3)
+    Wg32 = torch.randn(E, I, J, generator=g) / I ** 0.5
+    Ws32 = torch.randn(E, J, I, generator=g) / J ** 0.5
+    X = dev(case["X"]).requires_grad_(True); Wg = dev(Wg32).requires_grad_(True); Ws = dev(Ws32).requires_grad_(True)
+    Ind = dev(case["Ind"])
+    Y = hk.ExpertGatherFunction.apply(X, Wg, Ind, out_type)
+    out = hk.ExpertScatterFunction.apply(Y, Ws, Ind, T, out_type)
+    assert Y.dtype == torch.bfloat16 and out.dtype == torch.bfloat16
+    out.backward(dev(case["dOut"]))
+    assert X.grad.dtype == torch.bfloat16 and Wg.grad.dtype == torch.float32 and Ws.grad.dtype == torch.float32
+    rnd = (lambda w: w.to(torch.bfloat16)) if out_type == torch.bfloat16 else (lambda w: w)
+    Wgn, Wsn = np64(rnd(Wg32)), np64(rnd(Ws32))
+    Indn = case["Ind"].numpy()
+    assert_close(Y, O.gather_forward(np64(case["X"]), Wgn, Indn), torch.bfloat16, "Y mixed")
+    assert_close(out, O.scatter_forward(np64(Y), Wsn, Indn, T), torch.bfloat16, "out mixed")
+    dYo, dWso = O.scatter_backward(np64(Y), Wsn, Indn, np64(case["dOut"]))
+    wtol = torch.bfloat16 if out_type == torch.bfloat16 else torch.float32
+    assert_close(Ws.grad, dWso, wtol, "dWs mixed")
+    dY = torch.from_numpy(dYo).to(torch.bfloat16)
+    dXo, dWgo = O.gather_backward(np64(case["X"]), Wgn, Indn, np64(dY))
+    assert_close(X.grad, dXo, torch.bfloat16, "dX mixed")
+    # dW_gather sees dY rounded to the compute type before it is used; the fp32 path keeps dY in fp32
+    if out_type == torch.bfloat16:
+        assert_close(Wg.grad, dWgo, torch.bfloat16, "dWg mixed")
+
+
+def test_modules_trace_through_torch_compile():
+    """gather -> scatter forward and backward through the modules under torch.compile (aot_eager, one graph): the custom ops
+    carry fake implementations and autograd formulas, so nothing falls back to eager or breaks the graph; results equal the
+    eager ones bit for bit.  Counterpart of the reference's registration glue (egs/triton_kernels.py:527-567)."""
+    B, T, E, K, I, J = 4, 64, 8, 16, 128, 64
+    case = make_case(71, B, T, E, K, I, J, torch.bfloat16)
+    gather = egs.ExpertGather(E, I, J).to(DEV, torch.bfloat16); scatter = egs.ExpertScatter(E, J, I).to(DEV, torch.bfloat16)
+    with torch.no_grad():
+        gather.W.copy_(case["Wg"]); scatter.W.copy_(case["Ws"])
+    Ind = dev(case["Ind"]); dOut = dev(case["dOut"])
+
+    def block(x):
+        return scatter(gather(x, Ind), Ind, T)
+
+    def run(fn):
+        for m in (gather, scatter):
+            m.W.grad = None
+        x = dev(case["X"]).requires_grad_(True)
+        out = fn(x)
+        out.backward(dOut)
+        return out.detach(), x.grad, gather.W.grad.clone(), scatter.W.grad.clone()
+
+    eager = run(block)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(block, backend="aot_eager", fullgraph=True))
+    for name, a, b in zip(("out", "dX", "dWg", "dWs"), eager, compiled):
+        assert torch.equal(a, b), f"{name}: compiled differs from eager"
+    assert_close(eager[0], O.scatter_forward(np64(gather(dev(case["X"]), Ind)), np64(case["Ws"]), case["Ind"].numpy(), T),
+                 torch.bfloat16, "compiled block")

@@ -130,3 +130,66 @@ def test_bench_refuses_more_than_one_gpu():
                          timeout=120)
     assert res.returncode != 0
     assert "one GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_compute_dtype_follows_the_reference_kernels():
+    # out_type float16 / bfloat16: both operands are cast to it (reference egs/triton_kernels.py:122-127);
+    # float32: operands stay as they are - a shared 16-bit type is multiplied in that type, mixed types meet in float32
+    f32, f16, bf16 = torch.float32, torch.float16, torch.bfloat16
+    t = lambda dt: torch.empty(1, dtype=dt)
+    assert hk._compute_dtype(bf16, t(f32), t(f32)) == bf16
+    assert hk._compute_dtype(bf16, t(bf16), t(f32)) == bf16
+    assert hk._compute_dtype(f16, t(bf16), t(f32)) == f16
+    assert hk._compute_dtype(f32, t(bf16), t(bf16)) == bf16
+    assert hk._compute_dtype(f32, t(bf16), t(f32)) == f32
+    assert hk._compute_dtype(f32, t(f16), t(bf16), t(f32)) == f32
+    assert hk._compute_dtype(f32, t(f32), t(f32)) == f32
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        hk._compute_dtype(torch.int32, t(f32), t(f32))
+    with pytest.raises(ValueError, match="Unknown dtype"):
+        hk._compute_dtype(f32, t(torch.float64), t(f32))
+
+
+def test_mixed_precision_shapes_and_dtypes_on_meta_tensors():
+    # bf16 activations with an fp32 parameter, as under autocast-style use of the reference: results in the activation's
+    # dtype, weight gradient in the parameter's dtype (reference egs/triton_kernels.py:375, :408-409)
+    X = torch.empty(2, 5, 8, device="meta", dtype=torch.bfloat16, requires_grad=True)
+    W = torch.empty(4, 8, 6, device="meta", dtype=torch.float32, requires_grad=True)
+    Ind = torch.empty(2, 4, 3, dtype=torch.int16, device="meta")
+    Y = hk.ExpertGatherFunction.apply(X, W, Ind, torch.bfloat16)
+    assert Y.dtype == torch.bfloat16
+    Y.sum().backward()
+    assert X.grad.dtype == torch.bfloat16 and W.grad.dtype == torch.float32
+
+
+def test_ops_are_differentiable_when_called_directly():
+    hk.create_kernels()
+    X = torch.empty(2, 5, 8, device="meta", requires_grad=True)
+    W = torch.empty(4, 8, 6, device="meta", requires_grad=True)
+    Ind = torch.empty(2, 4, 3, dtype=torch.int64, device="meta")
+    Y = torch.ops.egs_amd.expert_gather_forward_call_fn(X, W, Ind, torch.float32)
+    assert Y.requires_grad
+    Y.sum().backward()
+    assert X.grad.shape == X.shape and W.grad.shape == W.shape
+
+
+def test_reference_namespace_alias():
+    # the reference registers its ops as mylib::* (egs/triton_kernels.py:362); the alias is opt-in
+    hk.register_reference_namespace("mylib_alias_for_test")
+    hk.register_reference_namespace("mylib_alias_for_test")          # idempotent
+    ops = torch.ops.mylib_alias_for_test
+    X = torch.empty(2, 5, 8, device="meta"); W = torch.empty(4, 8, 6, device="meta")
+    Ind = torch.empty(2, 4, 3, dtype=torch.int64, device="meta")
+    assert ops.expert_gather_forward_call_fn(X, W, Ind, torch.float32).shape == (2, 4, 3, 6)
+    assert ops.expert_scatter_forward_call_fn(torch.empty(2, 4, 3, 6, device="meta"), torch.empty(4, 6, 8, device="meta"), Ind, 5,
+                                              torch.float32).shape == (2, 5, 8)
+
+
+def test_scratch_is_allocated_per_call():
+    # no buffer survives a call: nothing whose address a captured graph could keep after it has been freed or regrown
+    keep, ptr, n = hk._workspace(torch.device("cpu"), 0)
+    assert keep is None and ptr is None and n == 0
+    keep, ptr, n = hk._workspace(torch.device("cpu"), 1000)
+    assert keep.numel() == 1000 and ptr == keep.data_ptr() and n == 1000
+    assert not hasattr(hk, "_workspaces")
+    hk.release_workspaces()                                           # harmless no-op
