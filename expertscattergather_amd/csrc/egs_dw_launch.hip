@@ -27,8 +27,7 @@ int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *
     const uint64_t x_span = d->B > 0 && d->T > 0
         ? ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES : 0;
     const uint64_t y_span = (uint64_t)d->B * d->E * d->K * d->J * ES;
-    if (pl.big_ok && !g_force_generic && p.x_vec && p.y_vec && x_span < (1ull << 31) && y_span < (1ull << 31) &&
-        aligned_to(dW, 16)) {
+    if (dw_big_takes(pl, Xs, Ys, dW, d, ldx_b, ldx_t, act_dtype)) {
         DwDlParams q;
         q.d = p;
         q.d.i_tiles = pl.b_i_tiles; q.d.j_tiles = pl.b_j_tiles; q.d.S = pl.b_S; q.d.rows_per_split = pl.b_rows_per_split;

@@ -67,8 +67,21 @@ struct DwPlan {
     int s_i_tiles, s_j_tiles, s_S, s_rows_per_split;        // its plan
     bool big_ok;                                            // shape admits the direct-to-LDS kernel (256 x BQ tiles)
     int b_bq, b_i_tiles, b_j_tiles, b_S, b_rows_per_split;  // its plan
-    size_t bytes;                                           // workspace covering whichever runs
+    size_t bytes_general, bytes_small, bytes_big;           // workspace of each of the three split kernels (0: no splits)
 };
+
+// does the direct-to-LDS weight gradient (dw_dl_kernel) take these operands?
+inline bool dw_big_takes(const DwPlan &pl, const void *Xs, const void *Ys, const void *dW, const egs_dims *d, int64_t ldx_b,
+                         int64_t ldx_t, int act_dtype)
+{
+    if (!pl.big_ok || g_force_generic || d->B < 1 || d->T < 1) return false;
+    const int ES = elem_size(act_dtype);
+    const bool x_vec = aligned_to(Xs, 16) && (ldx_b * ES) % 16 == 0 && (ldx_t * ES) % 16 == 0;
+    const bool y_vec = aligned_to(Ys, 16) && ((int64_t)d->J * ES) % 16 == 0;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + (uint64_t)d->I) * ES;
+    const uint64_t y_span = (uint64_t)d->B * d->E * d->K * d->J * ES;
+    return x_vec && y_vec && x_span < (1ull << 31) && y_span < (1ull << 31) && aligned_to(dW, 16);
+}
 
 
 // ---- egs_rows_launch.hip: tiled rows x weight products (general and direct-to-LDS kernels)

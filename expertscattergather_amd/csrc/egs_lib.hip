@@ -105,19 +105,20 @@ struct ScatterPlan {
     size_t bytes;
 };
 
-// Workspace of the GEMM-scatter: routing table (segment offsets, picks in token order, scratch
-// ranks, optional global counters) and the product rows in pick order.
-//   deterministic mode: product rows in fp32 -> fp32 accumulation with one final rounding;
-//   atomic ("fast") mode: with 16-bit element types the product rows are kept in the element
-//   type (half the traffic, one extra rounding per pick; the summation
-//   order is still fixed); fp32 uses global atomics on the output, no workspace.
-// The rows region is always sized for fp32.
-ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
+// Workspace of the GEMM-scatter, for the kernels that will run:
+//   fp32 atomic mode and the one-kernel scatter of small experts (`fused`) need none;
+//   otherwise: routing table (segment offsets, picks in token order, scratch ranks, optional global counters),
+//   long-segment records and partial rows, and the product rows in pick order - fp32 in deterministic mode
+//   (fp32 accumulation with one final rounding), the element type in atomic ("fast") mode with 16-bit types
+//   (half the traffic, one extra rounding per pick; the summation order is still fixed).
+ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype, bool fused)
 {
     ScatterPlan pl;
     memset(&pl, 0, sizeof(pl));
     const size_t N = (size_t)d->E * d->K;
     if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) return pl;
+    if (fused) return pl;
+    const size_t row_es = (mode == EGS_SCATTER_DETERMINISTIC || act_dtype == EGS_F32) ? 4 : (size_t)elem_size(act_dtype);
     size_t at = 0;
     pl.seg_off_at = at; at += align_up((size_t)d->B * ((size_t)d->T + 1) * 4, 256);
     pl.perm_at = at;    at += align_up((size_t)d->B * N * 4, 256);
@@ -126,7 +127,7 @@ ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype)
     // long segments (tokens picked more than kLongSegment times): records and fp32 partial rows
     pl.long_tab_at = at;  at += align_up((size_t)d->B * long_tab_stride((int)N) * 4, 256);
     pl.long_part_at = at; at += align_up((size_t)d->B * long_max_slots((int)N) * d->I * 4, 256);
-    pl.rows_at = at;    at += align_up((size_t)d->B * N * d->I * 4, 256);
+    pl.rows_at = at;    at += align_up((size_t)d->B * N * d->I * row_es, 256);
     pl.bytes = at;
     return pl;
 }
@@ -151,7 +152,7 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
     S = Me > 0 ? (Me + rows - 1) / rows : 1;
     pl.S = (int)S;
     pl.rows_per_split = (int)rows;
-    pl.bytes = S > 1 ? align_up((size_t)S * d->E * d->I * d->J * 4, 256) : 0;
+    pl.bytes_general = S > 1 ? align_up((size_t)S * d->E * d->I * d->J * 4, 256) : 0;
 
     // large 16-bit shapes: 256 x 256 (or 256 x 128) tiles, 64-row slabs, splits only to give every CU a workgroup
     // (C4: 2 splits 42 us, 4 splits 49 us, none 50 us)
@@ -170,8 +171,7 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
         s3 = (Me + r3 - 1) / r3;
         pl.b_S = (int)s3;
         pl.b_rows_per_split = (int)r3;
-        const size_t b3 = s3 > 1 ? align_up((size_t)s3 * d->E * d->I * d->J * 4, 256) : 0;
-        if (b3 > pl.bytes) pl.bytes = b3;
+        pl.bytes_big = s3 > 1 ? align_up((size_t)s3 * d->E * d->I * d->J * 4, 256) : 0;
     }
 
     // small experts: 64 x 64 tiles, up to 1024 picks per workgroup, enough workgroups to cover the device
@@ -189,8 +189,7 @@ DwPlan plan_dw(const egs_dims *d, int act_dtype)
         s2 = (Me + r2 - 1) / r2;
         pl.s_S = (int)s2;
         pl.s_rows_per_split = (int)r2;
-        const size_t b2 = s2 > 1 ? align_up((size_t)s2 * d->E * d->I * d->J * 4, 256) : 0;
-        if (b2 > pl.bytes) pl.bytes = b2;
+        pl.bytes_small = s2 > 1 ? align_up((size_t)s2 * d->E * d->I * d->J * 4, 256) : 0;
     }
     return pl;
 }
@@ -587,24 +586,32 @@ int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int 
     }
 }
 
-// GEMM-scatter of small experts in one kernel (product rows stay in LDS); `used` reports whether the
-// shape qualified.  Both scatter modes take it: it is bitwise reproducible and needs no workspace.
-int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
-                  int w_layout, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s, bool &used)
+// Does the one-kernel scatter of small experts (product rows stay in LDS, no workspace) take this problem?
+bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype)
 {
-    used = false;
     const int R = d->J, N = d->I;
     const int64_t NP = (int64_t)d->E * d->K;
-    if (g_force_generic || !(R == 32 || R == 64 || (R == 128 && act_dtype != EGS_F32))) return EGS_OK;
+    if (g_force_generic || !(R == 32 || R == 64 || (R == 128 && act_dtype != EGS_F32))) return false;
     const int ES = elem_size(act_dtype);
-    if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 1024 || d->T < 1 || d->B < 1) return EGS_OK;
-    const size_t lds = scatter_fused_lds(d->T, (int)NP);
-    if (lds > 156 * 1024) return EGS_OK;
-    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 16)) return EGS_OK;
-    if ((uint64_t)d->B * NP * R * ES > kSpan32 || (uint64_t)d->E * R * N * ES > kSpan32) return EGS_OK;
+    if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 1024 || d->T < 1 || d->B < 1) return false;
+    if (scatter_fused_lds(d->T, (int)NP) > 156 * 1024) return false;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 16)) return false;
+    if ((uint64_t)d->B * NP * R * ES > kSpan32 || (uint64_t)d->E * R * N * ES > kSpan32) return false;
     const int slices = N / kFusedCols;
     const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
-    if (blocks > INT32_MAX / 2 || (int64_t)d->B * slices < 8) return EGS_OK;        // too few workgroups to be worth it
+    return blocks <= INT32_MAX / 2 && (int64_t)d->B * slices >= 8;      // fewer workgroups are not worth it
+}
+
+// GEMM-scatter of small experts in one kernel; the caller has checked scatter_fused_takes().  Both scatter modes
+// take it: it is bitwise reproducible and needs no workspace.
+int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
+                  int w_layout, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
+{
+    const int R = d->J, N = d->I;
+    const int64_t NP = (int64_t)d->E * d->K;
+    const size_t lds = scatter_fused_lds(d->T, (int)NP);
+    const int slices = N / kFusedCols;
+    const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
     ScatterFusedParams p;
     memset(&p, 0, sizeof(p));
     p.A = (const char *)Y; p.W = (const char *)W; p.Ind = Ind; p.out = (char *)Out;
@@ -613,7 +620,6 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.slices = slices;
     p.perm_at = (int32_t)(NP * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
-    used = true;
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
     if (act_dtype == EGS_F32)
         return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, nullptr, s)
@@ -623,6 +629,34 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
                       : launch_scatter_fused_ks<ElemF16, false>(p, R, lds, (int)blocks, dw, dwt, s);
     return nmajor ? launch_scatter_fused_ks<ElemBF16, true>(p, R, lds, (int)blocks, dw, dwt, s)
                   : launch_scatter_fused_ks<ElemBF16, false>(p, R, lds, (int)blocks, dw, dwt, s);
+}
+
+// Which weight-gradient kernel takes these operands, and the workspace it needs.  egs_workspace_bytes asks with
+// stand-in operands (dense, 16-byte aligned); the entry points ask with the real ones, so what is planned and what
+// runs agree by construction.
+enum DwPath { DW_TILE, DW_SMALL, DW_BIG, DW_GENERAL };
+struct DwChoice { DwPath path; size_t bytes; };
+
+DwChoice dw_choose(const void *Xs, const void *Ys, void *dW, const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype,
+                   const DwPlan &pl)
+{
+    DwTileJob tj;
+    if (make_dw_tile(Xs, Ys, nullptr, dW, d, ldx_b, ldx_t, act_dtype, act_dtype, 0, 0, tj)) return {DW_TILE, 0};
+    SmallDwJob sj;
+    if (make_dw_small(Xs, Ys, nullptr, dW, nullptr, d, ldx_b, ldx_t, act_dtype, act_dtype, 0, 0, pl, sj)) return {DW_SMALL, pl.bytes_small};
+    if (dw_big_takes(pl, Xs, Ys, dW, d, ldx_b, ldx_t, act_dtype)) return {DW_BIG, pl.bytes_big};
+    return {DW_GENERAL, pl.bytes_general};
+}
+
+void *const kStandInPtr = (void *)(uintptr_t)4096;      // aligned, never dereferenced
+
+size_t dw_bytes_planned(const egs_dims *d, int act_dtype)
+{
+    return dw_choose(kStandInPtr, kStandInPtr, kStandInPtr, d, (int64_t)d->T * d->I, d->I, act_dtype, plan_dw(d, act_dtype)).bytes;
+}
+size_t scatter_bytes_planned(const egs_dims *d, int mode, int act_dtype)
+{
+    return plan_scatter(d, mode, act_dtype, scatter_fused_takes(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype)).bytes;
 }
 
 // ------------------------------------------------------------------------------ implementations
@@ -665,7 +699,8 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     const int ES = elem_size(act_dtype);
     const size_t out_elems = (size_t)d->B * d->T * d->I;
     if (out_elems == 0) return EGS_OK;
-    const ScatterPlan pl = plan_scatter(d, mode, act_dtype);
+    const bool fused = scatter_fused_takes(Y, W, Out, d, act_dtype);
+    const ScatterPlan pl = plan_scatter(d, mode, act_dtype, fused);
     char *ws = (char *)workspace;
     const int N = d->E * d->K;
 
@@ -694,11 +729,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         return rows_gemm_scatter(p, act_dtype, w_trans, EPI_ATOMIC_F32, s);
     }
 
-    {   // small experts: everything in one kernel
-        bool used = false;
-        const int rc_fused = scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s, used);
-        if (used) return rc_fused;
-    }
+    if (fused) return scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s);    // small experts: one kernel
 
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
     // gather-and-sum per token that writes every output row exactly once
@@ -777,17 +808,22 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
             int64_t ldx_b, int64_t ldx_t, int act_dtype, int out_dtype, int ind_dtype, int dw_layout, hipStream_t s)
 {
     if ((size_t)d->E * d->I * d->J == 0) return EGS_OK;
-    const DwPlan pl = plan_dw(d, act_dtype);
-    DwTileJob jt;
-    if (make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt))
+    DwPlan pl = plan_dw(d, act_dtype);
+    switch (dw_choose(Xs, Ys, dW, d, ldx_b, ldx_t, act_dtype, pl).path) {
+    case DW_TILE: {
+        DwTileJob jt;
+        make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt);
         return launch_dw_tile_alone(jt, s);
-    SmallDwJob j;
-    if (make_dw_small(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, j)) {
-        int rc = launch_dw_small_alone(j, s);
-        if (rc != EGS_OK) return rc;
-        return launch_dw_reduce4(j, s);
     }
-    return dw_general(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, s);
+    case DW_SMALL: {
+        SmallDwJob j;
+        make_dw_small(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, j);
+        const int rc = launch_dw_small_alone(j, s);
+        return rc != EGS_OK ? rc : launch_dw_reduce4(j, s);
+    }
+    default:
+        return dw_general(Xs, Ys, Ind, dW, workspace, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, pl, s);
+    }
 }
 
 // ------------------------------------------------------------------------------ validation
@@ -830,7 +866,7 @@ int validate_scatter(const void *Y, const void *W, const void *Ind, const void *
     const size_t picks = (size_t)d->B * d->E * d->K;
     if (picks > 0 && Ind == nullptr) return EGS_ERR_NULL_POINTER;
     if (picks > 0 && d->J > 0 && (Y == nullptr || W == nullptr)) return EGS_ERR_NULL_POINTER;
-    const size_t need = plan_scatter(d, mode, act_dtype).bytes;
+    const size_t need = plan_scatter(d, mode, act_dtype, scatter_fused_takes(Y, W, Out, d, act_dtype)).bytes;
     if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return EGS_ERR_WORKSPACE;
     if (need > 0 && !aligned_to(workspace, 256)) return EGS_ERR_ALIGNMENT;
     const int ES = elem_size(act_dtype);
@@ -852,7 +888,7 @@ int validate_dw(const void *Xs, const void *Ys, const void *Ind, const void *dW,
     const size_t picks = (size_t)d->B * d->K;
     if (picks > 0 && (Xs == nullptr || Ys == nullptr || Ind == nullptr)) return EGS_ERR_NULL_POINTER;
     if (picks > 0 && d->T > 0 && (ldx_t < d->I || (d->B > 1 && ldx_b < 0))) return EGS_ERR_BAD_STRIDE;
-    const size_t need = plan_dw(d, act_dtype).bytes;
+    const size_t need = picks > 0 ? dw_choose(Xs, Ys, const_cast<void *>(dW), d, ldx_b, ldx_t, act_dtype, plan_dw(d, act_dtype)).bytes : 0;
     if (need > 0 && (workspace == nullptr || workspace_bytes < need)) return EGS_ERR_WORKSPACE;
     if (need > 0 && !aligned_to(workspace, 256)) return EGS_ERR_ALIGNMENT;
     const int ES = elem_size(act_dtype);
@@ -896,10 +932,10 @@ size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
     if (!mode_ok(mode)) mode = EGS_SCATTER_DETERMINISTIC;
     switch (op) {
     case EGS_OP_GATHER_GEMM: return 0;
-    case EGS_OP_GEMM_SCATTER: return plan_scatter(d, mode, act_dtype).bytes;
-    case EGS_OP_DW: return plan_dw(d, act_dtype).bytes;
-    case EGS_OP_GATHER_BACKWARD: return plan_scatter(d, mode, act_dtype).bytes + plan_dw(d, act_dtype).bytes;
-    case EGS_OP_SCATTER_BACKWARD: return plan_dw(d, act_dtype).bytes;
+    case EGS_OP_GEMM_SCATTER: return scatter_bytes_planned(d, mode, act_dtype);
+    case EGS_OP_DW: return dw_bytes_planned(d, act_dtype);
+    case EGS_OP_GATHER_BACKWARD: return scatter_bytes_planned(d, mode, act_dtype) + dw_bytes_planned(d, act_dtype);
+    case EGS_OP_SCATTER_BACKWARD: return dw_bytes_planned(d, act_dtype);
     default: return 0;
     }
 }
@@ -944,7 +980,8 @@ int egs_dw_builtin_scratch(const void *Xsrc, const void *Ysrc, const void *Ind, 
     int rc = check_dims(d);
     if (rc != EGS_OK) return rc;
     if (!act_dtype_ok(act_dtype)) return EGS_ERR_BAD_DTYPE;
-    const size_t need = plan_dw(d, act_dtype).bytes;
+    if (!layout_ok(dw_layout)) return EGS_ERR_BAD_LAYOUT;
+    const size_t need = dw_choose(Xsrc, Ysrc, dW, d, ldx_b, ldx_t, act_dtype, plan_dw(d, act_dtype)).bytes;
     if (need > (size_t)EGS_BUILTIN_SCRATCH_BYTES) return EGS_ERR_SCRATCH_LIMIT;
     // the remaining checks are those of egs_dw; the stand-in address only has to look like a valid workspace
     rc = validate_dw(Xsrc, Ysrc, Ind, dW, need > 0 ? (const void *)(uintptr_t)256 : nullptr, need, d, ldx_b, ldx_t, act_dtype,
@@ -979,8 +1016,10 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     if (rc != EGS_OK) return rc;
     if (!act_dtype_ok(dtype)) return EGS_ERR_BAD_DTYPE;
     if (!mode_ok(mode)) return EGS_ERR_BAD_MODE;
-    const size_t ws_scatter = plan_scatter(d, mode, dtype).bytes;
-    const size_t ws_dw = plan_dw(d, dtype).bytes;
+    if (grad_X == nullptr && (size_t)d->B * d->T * d->I > 0) return EGS_ERR_NULL_POINTER;
+    const size_t ws_scatter = plan_scatter(d, mode, dtype, scatter_fused_takes(grad_Y, W, grad_X, d, dtype)).bytes;
+    const size_t ws_dw = (size_t)d->B * d->K > 0 && (size_t)d->E * d->I * d->J > 0 && grad_W != nullptr
+        ? dw_choose(X, grad_Y, grad_W, d, ldx_b, ldx_t, dtype, plan_dw(d, dtype)).bytes : 0;
     if (ws_scatter + ws_dw > 0 && (workspace == nullptr || workspace_bytes < ws_scatter + ws_dw)) return EGS_ERR_WORKSPACE;
     // validate both halves before enqueuing anything
     rc = validate_scatter(grad_Y, W, Ind, grad_X, workspace, ws_scatter, d, dtype, ind_dtype, EGS_W_EIJ, mode);

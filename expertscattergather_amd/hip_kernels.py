@@ -133,6 +133,14 @@ def release_workspaces() -> None:
     allocated per call, so there is nothing to release."""
 
 
+def _dense16(t: torch.Tensor) -> torch.Tensor:
+    """Contiguous and starting on a 16-byte boundary.  egs_workspace_bytes() sizes the scratch for operands like that
+    (they take the specialised kernels); a view that starts at an odd element offset is copied rather than sent down
+    the general kernels with a workspace sized for the others."""
+    t = t.contiguous()
+    return t.clone() if t.data_ptr() % 16 else t
+
+
 def _rows_source(X: torch.Tensor):
     """[B,T,I] tensor -> (tensor with unit inner stride, batch stride, token stride)."""
     if X.stride(2) != 1 and X.shape[2] > 1:
@@ -140,8 +148,13 @@ def _rows_source(X: torch.Tensor):
     B, T, I = X.shape
     ld_t = X.stride(1) if T > 1 else max(I, 1)
     ld_b = X.stride(0) if B > 1 else ld_t * max(T, 1)
-    if ld_t < I or ld_b < 0:
+    es = X.element_size()
+    if ld_t < I or ld_b < 0 or ((I * es) % 16 == 0 and ((ld_t * es) % 16 or (ld_b * es) % 16)):
+        # overlapping rows, or strides that would take rows off the 16-byte grid their width allows
         X = X.contiguous()
+        ld_t, ld_b = I, T * I
+    if X.data_ptr() % 16:
+        X = X.contiguous().clone() if not X.is_contiguous() else X.clone()
         ld_t, ld_b = I, T * I
     return X, ld_b, ld_t
 
@@ -190,7 +203,7 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     B, E, K, I, J = _check_shapes(X, W, Ind, None, True)
     res_dtype = X.dtype
     X, ld_b, ld_t = _rows_source(X.to(ct))
-    W = W.to(ct).contiguous(); Ind = Ind.contiguous()
+    W = _dense16(W.to(ct)); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
     with _on_device(dev):
@@ -206,7 +219,7 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     B, E, K, I, J = _check_shapes(X, W, Ind, grad_output, True)
     x_dtype, w_dtype = X.dtype, W.dtype
     X, ld_b, ld_t = _rows_source(X.to(ct))
-    W = W.to(ct).contiguous(); Ind = Ind.contiguous(); grad_output = grad_output.to(ct).contiguous()
+    W = _dense16(W.to(ct)); Ind = Ind.contiguous(); grad_output = _dense16(grad_output.to(ct))
     T = X.shape[1]
     grad_X = torch.empty((B, T, I), device=dev, dtype=ct)
     grad_W = torch.empty((E, I, J), device=dev, dtype=ct)
@@ -231,7 +244,7 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     if T < 0:
         raise ValueError("T must be non-negative")
     res_dtype = Y.dtype
-    Y = Y.to(ct).contiguous(); W = W.to(ct).contiguous(); Ind = Ind.contiguous()
+    Y = _dense16(Y.to(ct)); W = _dense16(W.to(ct)); Ind = Ind.contiguous()
     out = torch.empty((B, T, I), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
@@ -251,7 +264,7 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
     B, E, K, I, J = _check_shapes(grad_X, W, Ind, Y, False)
     y_dtype, w_dtype = Y.dtype, W.dtype
     grad_X, ld_b, ld_t = _rows_source(grad_X.to(ct))
-    Y = Y.to(ct).contiguous(); W = W.to(ct).contiguous(); Ind = Ind.contiguous()
+    Y = _dense16(Y.to(ct)); W = _dense16(W.to(ct)); Ind = Ind.contiguous()
     T = grad_X.shape[1]
     grad_Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     grad_W = torch.empty((E, J, I), device=dev, dtype=ct)

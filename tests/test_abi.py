@@ -108,16 +108,28 @@ def test_builtin_scratch_entry_point_checks_sizes_first(lib):
 
 
 def test_workspace_sizes_are_consistent(lib):
-    d = _abi.Dims(64, 256, 32, 32, 128, 64)
     wb = lib.egs_workspace_bytes
-    assert wb(_abi.OP_GATHER_GEMM, 0, d, 2) == 0
-    det, dw = wb(_abi.OP_GEMM_SCATTER, 0, d, 2), wb(_abi.OP_DW, 0, d, 2)
-    assert det >= 64 * 32 * 32 * 128 * 4                                     # fp32 product rows
-    assert wb(_abi.OP_GATHER_BACKWARD, 0, d, 2) == det + dw
-    assert wb(_abi.OP_SCATTER_BACKWARD, 0, d, 2) == dw
-    assert wb(_abi.OP_GEMM_SCATTER, 1, d, 0) == 0                             # fp32 atomic mode adds into the output
+    # the default shape in bf16 runs on kernels that need no scratch at all: the one-kernel scatter keeps its product rows
+    # in LDS and the one-pass weight gradient has no partial sums
+    d = _abi.Dims(64, 256, 32, 32, 128, 64)
+    for op in (_abi.OP_GATHER_GEMM, _abi.OP_GEMM_SCATTER, _abi.OP_DW, _abi.OP_GATHER_BACKWARD, _abi.OP_SCATTER_BACKWARD):
+        assert wb(op, 0, d, _abi.BF16) == 0 and wb(op, 1, d, _abi.BF16) == 0
+    # more picks per batch element than the one-kernel scatter holds: routing table + fp32 product rows (deterministic) or
+    # rows in the element type (atomic mode with a 16-bit type); fewer experts than the one-pass weight gradient wants: splits
+    d = _abi.Dims(16, 256, 8, 256, 128, 64)
+    rows = 16 * 8 * 256 * 128
+    det, fast, dw = wb(_abi.OP_GEMM_SCATTER, 0, d, _abi.BF16), wb(_abi.OP_GEMM_SCATTER, 1, d, _abi.BF16), wb(_abi.OP_DW, 0, d, _abi.BF16)
+    assert rows * 4 <= det <= rows * 4 * 1.1 and rows * 2 <= fast <= rows * 2 * 1.1 and dw > 0
+    assert wb(_abi.OP_GATHER_BACKWARD, 0, d, _abi.BF16) == det + dw
+    assert wb(_abi.OP_SCATTER_BACKWARD, 0, d, _abi.BF16) == dw
+    assert wb(_abi.OP_GEMM_SCATTER, 1, d, _abi.F32) == 0                      # fp32 atomic mode adds into the output
     assert det % 256 == 0 and dw % 256 == 0
     assert wb(99, 0, d, 2) == 0 and wb(_abi.OP_DW, 0, d, 9) == 0
+    # an entry point checks the workspace against the kernels its actual operands select: an output that is not
+    # 16-byte aligned cannot take the one-kernel scatter and is refused without the general path's workspace
+    d = _abi.Dims(64, 256, 32, 32, 128, 64)
+    p = 0x1000
+    assert lib.egs_gemm_scatter(p, p, p, p + 2, None, 0, d, _abi.BF16, _abi.IND_I64, _abi.W_EJI, 0, None) == -6
 
 
 def test_check_raises_like_the_reference():
