@@ -7,9 +7,10 @@ dW_scatter) -> gather backward (dX, dW_gather), i.e. the six kernel-equivalents 
 autograd forward+backward.  Inputs are resident in HBM before the timed region starts.
 
 Prints ONE JSON line.  `value` is microseconds per step (lower is better); `roofline`
-describes the dominant kernel (algorithmic bytes / its average launch duration, measured
-with HIP events on the launch stream); `cpu_baseline` is the torch port of the reference's
-baselines timed on the host cores.
+describes the dominant launch of the step, the one that takes the most time (algorithmic bytes
+or flops / its average duration, measured with HIP events on the launch stream, warm and with
+the caches flushed), `roofline_per_launch` every launch; `cpu_baseline` is the torch port of
+the reference's baselines timed on the host cores.
 """
 from __future__ import annotations
 
@@ -27,14 +28,33 @@ HBM_PEAK_GBPS = 8000.0       # MI355X HBM3E, published
 # MI355X dense matrix peaks (TFLOP/s) of the arithmetic each configuration multiplies in
 MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0, "fp8": 5000.0}
 
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# runs of `bench.py --pmc-probe` scaled by a 64 MiB copy (summary: profiles/rows_small_gather_c2_traffic.md).
-# Counters cannot be read from inside this process, so the figure is the recorded one.
-MEASURED_TRAFFIC_BYTES = {("C2", "gather_gemm"): 17349000,        # profiles/rows_small_gather_c2_traffic.md
-                          ("C3", "gather_gemm"): 693100000,       # profiles/rows_gemm_dl_gather_c3_counters.md
-                          ("C1", "gather_gemm"): 46310000,        # profiles/gather_traffic_c1_c4_c5.md
-                          ("C4", "gather_gemm"): 80920000,
-                          ("C5", "gather_gemm"): 2922340000}
+PROFILES = os.path.join(ROOT, "profiles")
+
+# kernel (as rocprofv3 names it) behind each launch of the path, per workload; where a call runs several kernels
+# the one that takes most of its time is named and the others are listed in the profile summaries
+LAUNCH_KERNELS = {
+    "C2": {"expert_gather_forward": "rows_small_kernel", "expert_scatter_forward": "scatter_fused_kernel",
+           "expert_scatter_backward": "rows_dw_tile_kernel", "expert_gather_backward": "scatter_fused_dwtile_kernel"},
+    "C1": {"expert_gather_forward": "rows_gemm_kernel", "expert_scatter_forward": "scatter_fused_kernel"},
+    "C3": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel",
+           "expert_scatter_backward": "rows_gemm_dl_kernel + dw_dl_kernel", "expert_gather_backward": "rows_gemm_dl_kernel + segment_sum_kernel + dw_dl_kernel"},
+    "C4": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel",
+           "expert_scatter_backward": "rows_gemm_dl_kernel + dw_dl_kernel", "expert_gather_backward": "rows_gemm_dl_kernel + segment_sum_kernel + dw_dl_kernel"},
+    "C5": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel"},
+}
+
+
+def recorded_traffic():
+    """HBM-side bytes per launch from the rocprofv3 --pmc summaries under profiles/ (FETCH_SIZE + WRITE_SIZE of
+    `bench.py --pmc-probe` runs, each scaled by what the same counter reads for a 64 MiB copy).  Counters cannot be read
+    from inside this process, so the figures are the recorded ones: lines `traffic <workload> <launch> <bytes>`."""
+    import glob
+    import re
+    found = {}
+    for path in sorted(glob.glob(os.path.join(PROFILES, "*.md")) + glob.glob(os.path.join(PROFILES, "*.txt"))):
+        for m in re.finditer(r"^\s*traffic (\S+) (\S+) (\d+)\s*$", open(path).read(), flags=re.M):
+            found[(m.group(1), m.group(2))] = {"bytes": int(m.group(3)), "source": os.path.relpath(path, ROOT)}
+    return found
 
 
 def parse_args():
@@ -49,7 +69,7 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--kernel-reps", type=int, default=200, help="launches per kernel for the per-kernel timing")
-    ap.add_argument("--cold", action="store_true", help="also time each kernel with the caches flushed between launches")
+    ap.add_argument("--no-cold", action="store_true", help="skip the timing of each launch with the caches flushed in between")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch a 64 MiB device copy (3x) and one entry point of the path (5x), for rocprofv3 --pmc runs")
     ap.add_argument("--probe-kernel", default="gather", choices=["gather", "scatter", "dw", "scatter_bwd", "gather_bwd"],
@@ -174,37 +194,52 @@ def main():
     use_graph = graph_s is not None and graph_s <= eager_s
     step_s = graph_s if use_graph else eager_s
 
-    # ------------------------------------------------------------------ per-kernel timing (HIP events)
+    # ------------------------------------------------------------------ per-launch timing (HIP events)
+    # Every launch of the step through the C ABI, back to back on torch's current stream (the stream the launches are
+    # enqueued on), bracketed by HIP events; and once more with the caches flushed before every launch.
     act = 2 if cfg.dtype != torch.float32 else 4
     lib = _abi.lib()
     d = _abi.Dims(B, T, E, K, I, J)
     dt = hk.dtype_to_type_id(cfg.dtype)
     stream = torch.cuda.current_stream().cuda_stream
-    Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32) if not fp8 else hk.expert_gather_fp8w_forward(X, Wq, Wscale, Ind)
     out = torch.empty(B, T, I, device=dev, dtype=cfg.dtype)
-    dWbuf = torch.empty(E, I, J, device=dev, dtype=cfg.dtype)
+    dYb, dXb = torch.empty_like(Y), torch.empty(B, T, I, device=dev, dtype=cfg.dtype)
+    dWg_b, dWs_b = torch.empty(E, I, J, device=dev, dtype=cfg.dtype), torch.empty(E, J, I, device=dev, dtype=cfg.dtype)
     mode = 0 if hk.get_scatter_mode() == "deterministic" else 1
-    ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
+    ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     f8ws_bytes = lib.egs_gather_gemm_fp8act_workspace_bytes(d) if fp8_act else 0
     f8ws = torch.empty(max(f8ws_bytes, 256), dtype=torch.uint8, device=dev)
+    I64 = _abi.IND_I64
 
     def k_gather():
         if fp8_act:     # row quantiser + fp8 x fp8 product: both launches are part of the call
             return lib.egs_gather_gemm_fp8act(X.data_ptr(), Wq.data_ptr(), Wscale.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
-                                              f8ws.data_ptr(), f8ws_bytes, d, T * I, I, 2, stream)
+                                              f8ws.data_ptr(), f8ws_bytes, d, T * I, I, I64, stream)
         if fp8:
-            return lib.egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), Wscale.data_ptr(), d, T * I, I, dt, 3, 2, 0, stream)
-        return lib.egs_gather_gemm(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), None, d, T * I, I, dt, dt, 2, 0, stream)
+            return lib.egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), Wscale.data_ptr(), d, T * I, I, dt,
+                                       _abi.FP8_E4M3, I64, _abi.W_EIJ, stream)
+        return lib.egs_expert_gather_forward(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d, T * I, I, dt, I64, stream)
 
     def k_scatter():
-        return lib.egs_gemm_scatter(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, d, dt, 2, 1, mode, stream)
+        return lib.egs_expert_scatter_forward(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, d,
+                                              dt, I64, mode, stream)
+
+    def k_scatter_bwd():
+        return lib.egs_expert_scatter_backward(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), dOut.data_ptr(), dYb.data_ptr(),
+                                               dWs_b.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, I64, stream)
+
+    def k_gather_bwd():
+        return lib.egs_expert_gather_backward(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), dYb.data_ptr(), dXb.data_ptr(),
+                                              dWg_b.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, I64, mode, stream)
 
     def k_dw():
-        return lib.egs_dw(X.data_ptr(), Y.data_ptr(), Ind.data_ptr(), dWbuf.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, dt, 2, 0, stream)
+        return lib.egs_dw(X.data_ptr(), Y.data_ptr(), Ind.data_ptr(), dWg_b.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, dt,
+                          I64, _abi.W_EIJ, stream)
 
     # a buffer larger than the 256 MB Infinity Cache, rewritten between launches for the cold numbers
-    flush = torch.empty(640 << 20, dtype=torch.uint8, device=dev) if args.cold else None
+    flush = None if args.no_cold else torch.empty(640 << 20, dtype=torch.uint8, device=dev)
 
     def time_kernel(fn, reps):
         for _ in range(5):
@@ -234,31 +269,45 @@ def main():
     gemm_bytes = wl.algorithmic_bytes(dims, act)
     gather_bytes = wl.algorithmic_bytes(dims, act, w_bytes=1, fp8_scales=True) if fp8 else gemm_bytes
     dw_bytes = wl.algorithmic_bytes(dims, act, dw=True)
+    kflops = wl.flops(dims)
     reps = args.kernel_reps if args.config in ("C1", "C2") else max(5, args.kernel_reps // 10)
-    kernels = {
-        "gather_gemm": (time_kernel(k_gather, reps), gather_bytes),
-        "gemm_scatter": (time_kernel(k_scatter, reps), gemm_bytes),
-    }
+    # launch -> (function, algorithmic bytes, flops): the backward calls compute two kernel-equivalents each
+    launches = {"expert_gather_forward": (k_gather, gather_bytes, kflops), "expert_scatter_forward": (k_scatter, gemm_bytes, kflops)}
     if not fwd_only:
-        kernels["dw"] = (time_kernel(k_dw, reps), dw_bytes)
-    cold = None
-    if args.cold:
-        cold = {"gather_gemm": time_kernel_cold(k_gather, 10), "gemm_scatter": time_kernel_cold(k_scatter, 10)}
-        if not fwd_only:
-            cold["dw"] = time_kernel_cold(k_dw, 10)
-    # gather_gemm is the kernel the whole path is named after and runs twice per step
-    dom = "gather_gemm"
-    dom_s, dom_bytes = kernels[dom]
+        launches["expert_scatter_backward"] = (k_scatter_bwd, gemm_bytes + dw_bytes, 2 * kflops)
+        launches["expert_gather_backward"] = (k_gather_bwd, gemm_bytes + dw_bytes, 2 * kflops)
+    warm = {name: time_kernel(fn, reps) for name, (fn, _, _) in launches.items()}
+    cold = None if flush is None else {name: time_kernel_cold(fn, 10) for name, (fn, _, _) in launches.items()}
+    dw_alone_s = None if fwd_only else time_kernel(k_dw, reps)
+    del flush
     n_equiv = 2 if fwd_only else 6
     chain_bytes = (gather_bytes + gemm_bytes) if fwd_only else 4 * gemm_bytes + 2 * dw_bytes
-    kflops = wl.flops(dims)
     chain_flops = n_equiv * kflops
     dtype_name = "bf16" if cfg.dtype == torch.bfloat16 else ("f16" if cfg.dtype == torch.float16 else "f32")
     mfma_peak = MFMA_PEAK_TFLOPS["fp8" if fp8_act else dtype_name]
-    # the roof that binds a kernel is the slower of "move the algorithmic bytes at 8 TB/s" and
-    # "do the flops at the dense matrix peak of the arithmetic type"
-    t_hbm, t_mfma = dom_bytes / (HBM_PEAK_GBPS * 1e9), kflops / (mfma_peak * 1e12)
-    bound = "hbm" if t_hbm >= t_mfma else "mfma"
+    traffic = recorded_traffic()
+
+    def roofline_of(name):
+        # the roof that binds a launch is the slower of "move its algorithmic bytes at 8 TB/s" and "do its flops at the
+        # dense matrix peak of the arithmetic type"
+        _, nbytes, nflops = launches[name]
+        t = warm[name]
+        t_hbm, t_mfma = nbytes / (HBM_PEAK_GBPS * 1e9), nflops / (mfma_peak * 1e12)
+        tr = traffic.get((args.config, name))
+        common = {"launch": name, "kernel": LAUNCH_KERNELS.get(args.config, {}).get(name), "avg_launch_us": round(t * 1e6, 3),
+                  "avg_launch_us_cold": None if cold is None else round(cold[name] * 1e6, 3),
+                  "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,
+                  "hbm_frac": round(nbytes / t * 1e-9 / HBM_PEAK_GBPS, 4), "mfma_frac": round(nflops / t * 1e-12 / mfma_peak, 4),
+                  "traffic": None if tr is None or fp8_act else tr["bytes"], "traffic_source": None if tr is None or fp8_act else tr["source"]}
+        if t_hbm >= t_mfma:
+            return {"bound": "hbm", "achieved": round(nbytes / t * 1e-9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(nbytes / t * 1e-9 / HBM_PEAK_GBPS, 4), **common}
+        return {"bound": "mfma", "achieved": round(nflops / t * 1e-12, 2), "peak": mfma_peak, "unit": "TFLOP/s",
+                "frac": round(nflops / t * 1e-12 / mfma_peak, 4), **common}
+
+    # the dominant launch is the one that takes most of a step (every launch runs once per step)
+    dom = max(warm, key=warm.get)
+    rooflines = {name: roofline_of(name) for name in launches}
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     cpu = None
@@ -315,21 +364,11 @@ def main():
         "step_tflops": round(chain_flops / step_s * 1e-12, 2),
         "eager_us_per_step": round(eager_s * 1e6, 2),
         "graph_us_per_step": None if graph_s is None else round(graph_s * 1e6, 2),
-        "kernel_us": {k: round(v[0] * 1e6, 2) for k, v in kernels.items()},
-        "kernel_us_cold": None if cold is None else {k: round(v * 1e6, 2) for k, v in cold.items()},
-        "kernel_hbm_gbps": {k: round(v[1] / v[0] * 1e-9, 1) for k, v in kernels.items()},
-        "kernel_hbm_frac": {k: round(v[1] / v[0] * 1e-9 / HBM_PEAK_GBPS, 4) for k, v in kernels.items()},
-        "kernel_tflops": {k: round(kflops / v[0] * 1e-12, 2) for k, v in kernels.items()},
-        "kernel_mfma_frac": {k: round(kflops / v[0] * 1e-12 / mfma_peak, 4) for k, v in kernels.items()},
-        "roofline": ({"bound": "hbm", "kernel": dom, "achieved": round(dom_bytes / dom_s * 1e-9, 1), "peak": HBM_PEAK_GBPS,
-                      "unit": "GB/s", "frac": round(dom_bytes / dom_s * 1e-9 / HBM_PEAK_GBPS, 4),
-                      "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
-                      "algorithmic_bytes": dom_bytes, "avg_launch_us": round(dom_s * 1e6, 3)}
-                     if bound == "hbm" else
-                     {"bound": "mfma", "kernel": dom, "achieved": round(kflops / dom_s * 1e-12, 2), "peak": mfma_peak,
-                      "unit": "TFLOP/s", "frac": round(kflops / dom_s * 1e-12 / mfma_peak, 4),
-                      "traffic": None if fp8_act else MEASURED_TRAFFIC_BYTES.get((args.config, dom)),
-                      "algorithmic_flops": kflops, "avg_launch_us": round(dom_s * 1e6, 3)}),
+        "launch_us": {k: round(v * 1e6, 2) for k, v in warm.items()},
+        "launch_us_cold": None if cold is None else {k: round(v * 1e6, 2) for k, v in cold.items()},
+        "dw_alone_us": None if dw_alone_s is None else round(dw_alone_s * 1e6, 2),
+        "roofline": rooflines[dom],
+        "roofline_per_launch": rooflines,
         "cpu_baseline": cpu,
     }
     print(json.dumps(result), flush=True)

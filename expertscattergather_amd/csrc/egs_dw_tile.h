@@ -141,10 +141,19 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
 
     // fragment addresses inside a piece ([32 picks][64 or YB bytes]): the lane points at pick 8 g + 4 h + a / 4 and the
     // four columns 4 (a % 4) of a 16-column group, and receives column a of picks 8 g + 4 h .. + 3
-    const int at0 = (g * 8 + (a >> 2)) * 64 + (a & 3) * 8, at1 = at0 + 4 * 64;
-    const int yat0 = (g * 8 + (a >> 2)) * YB + (a & 3) * 8, yat1 = yat0 + 4 * YB;
-    const int wr = (lane >> 2) * 64 + (lane & 3) * 16;
-    const int ywr = (lane / YL) * YB + (lane % YL) * 16;
+    // The 32-byte units of a row (one 16-column group each) are XOR-swizzled by the pick number so that the four picks
+    // a transpose read touches per 16 lanes fall on different banks: unit ^ (pick / 2 % 2) in the 64-byte rows, unit ^
+    // (pick % 4) in the 128-byte rows.  pick = 8 g + 4 h + a / 4 below, so the key depends on a / 4 only (and on h for
+    // the 64-byte rows, where at1 = at0 + 4 rows keeps pick / 2 % 2).
+    const int fr = a >> 2;                              // pick of the lane inside its group of four
+    const int xkey = (fr >> 1) & 1, ykey = YB == 64 ? (fr >> 1) & 1 : fr & 3;
+    const int at0 = (g * 8 + fr) * 64 + (a & 3) * 8, at1 = at0 + 4 * 64;
+    const int yat0 = (g * 8 + fr) * YB + (a & 3) * 8, yat1 = yat0 + 4 * YB;
+    // writers: lane holds chunk c (16 bytes = half a unit) of pick p
+    const int xp = lane >> 2, xcn = lane & 3;
+    const int wr = xp * 64 + (((xcn >> 1) ^ ((xp >> 1) & 1)) << 5) + (xcn & 1) * 16;
+    const int yp = lane / YL, ycn = lane % YL;
+    const int ywr = yp * YB + (((ycn >> 1) ^ (YB == 64 ? (yp >> 1) & 1 : yp & 3)) << 5) + (ycn & 1) * 16;
     // A step goes registers -> LDS tile (stage_write), LDS tile -> fragments (stage_read), fragments -> MFMAs.  The
     // loop is software-pipelined: the fragments of step s are requested first, then the registers of step s+1 are
     // dropped into the other tile (and refilled from the next chunk), then the MFMAs of step s run - so the LDS
@@ -160,12 +169,12 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
         const char *st = stage + (s & 1) * STG;
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
-            const u32x2 lo = lds_read_tr16(st + at0 + x * 32), hi = lds_read_tr16(st + at1 + x * 32);
+            const u32x2 lo = lds_read_tr16(st + at0 + ((x ^ xkey) << 5)), hi = lds_read_tr16(st + at1 + ((x ^ xkey) << 5));
             pf[x] = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
 #pragma unroll
         for (int y = 0; y < NY; ++y) {
-            const u32x2 lo = lds_read_tr16(st + 2048 + yat0 + y * 32), hi = lds_read_tr16(st + 2048 + yat1 + y * 32);
+            const u32x2 lo = lds_read_tr16(st + 2048 + yat0 + ((y ^ ykey) << 5)), hi = lds_read_tr16(st + 2048 + yat1 + ((y ^ ykey) << 5));
             qf[y] = u32x4{lo[0], lo[1], hi[0], hi[1]};
         }
     };

@@ -133,16 +133,37 @@ def release_workspaces() -> None:
     allocated per call, so there is nothing to release."""
 
 
-def _dense16(t: torch.Tensor) -> torch.Tensor:
-    """Contiguous and starting on a 16-byte boundary.  egs_workspace_bytes() sizes the scratch for operands like that
-    (they take the specialised kernels); a view that starts at an odd element offset is copied rather than sent down
-    the general kernels with a workspace sized for the others."""
-    t = t.contiguous()
+def _dense16(t: torch.Tensor, ct: torch.dtype) -> torch.Tensor:
+    """`t` in the compute dtype, contiguous and starting on a 16-byte boundary (nothing is done, and nothing paid, when
+    it already is).  egs_workspace_bytes() sizes the scratch for operands like that (they take the specialised
+    kernels); a view that starts at an odd element offset is copied rather than sent down the general kernels with
+    a workspace sized for the others."""
+    if t.dtype is ct and t.is_contiguous() and t.data_ptr() % 16 == 0:
+        return t
+    t = t.to(ct).contiguous()
     return t.clone() if t.data_ptr() % 16 else t
 
 
-def _rows_source(X: torch.Tensor):
-    """[B,T,I] tensor -> (tensor with unit inner stride, batch stride, token stride)."""
+_ws_sizes: dict = {}
+
+
+def _workspace_bytes(op: int, mode: int, dims: tuple, dt: int) -> int:
+    """egs_workspace_bytes(), remembered per problem: a pure function of its arguments, except for the test-suite's
+    switch egs_testing_force_generic, after which `_ws_sizes` has to be cleared."""
+    key = (op, mode, dims, dt)
+    n = _ws_sizes.get(key)
+    if n is None:
+        if len(_ws_sizes) > 4096:
+            _ws_sizes.clear()
+        n = _ws_sizes[key] = int(_abi.lib().egs_workspace_bytes(op, mode, _abi.Dims(*dims), dt))
+    return n
+
+
+def _rows_source(X: torch.Tensor, ct: torch.dtype):
+    """[B,T,I] tensor -> (tensor in the compute dtype with unit inner stride, batch stride, token stride)."""
+    if X.dtype is ct and X.is_contiguous() and X.data_ptr() % 16 == 0:
+        return X, X.shape[1] * X.shape[2], X.shape[2]
+    X = X.to(ct)
     if X.stride(2) != 1 and X.shape[2] > 1:
         X = X.contiguous()
     B, T, I = X.shape
@@ -186,14 +207,16 @@ def _compute_dtype(out_dtype: torch.dtype, *tensors: torch.Tensor) -> torch.dtyp
     operands that already share a 16-bit type are multiplied in that type (fp32 accumulation either way), and
     operands of different types meet in float32.  Results are returned in the dtype of the tensor they are the
     gradient of / the activation they continue (:375, :408-409, :457, :491-492)."""
-    dtype_to_type_id(out_dtype)
+    first = tensors[0].dtype
+    same = True
     for t in tensors:
         if t.dtype not in _FLOATS:
             raise ValueError("Unknown dtype")
-    if out_dtype != torch.float32:
-        return out_dtype
-    first = tensors[0].dtype
-    return first if all(t.dtype == first for t in tensors) else torch.float32
+        same = same and t.dtype is first
+    if out_dtype is torch.float32:
+        return first if same else torch.float32
+    dtype_to_type_id(out_dtype)
+    return out_dtype
 
 
 # ------------------------------------------------------------------------------ the four launchers
@@ -202,15 +225,16 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     dev = _require_gpu(X, W, Ind)
     B, E, K, I, J = _check_shapes(X, W, Ind, None, True)
     res_dtype = X.dtype
-    X, ld_b, ld_t = _rows_source(X.to(ct))
-    W = _dense16(W.to(ct)); Ind = Ind.contiguous()
+    X, ld_b, ld_t = _rows_source(X, ct)
+    W = _dense16(W, ct); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
     with _on_device(dev):
         rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
                                                   ld_b, ld_t, dtype_to_type_id(ct), _ind_type_id(Ind), _stream_ptr(dev))
-    _abi.check(rc, "expert_gather_forward_call")
-    return Y.to(res_dtype)
+    if rc:
+        _abi.check(rc, "expert_gather_forward_call")
+    return Y if res_dtype is ct else Y.to(res_dtype)
 
 
 def _gather_backward_impl(X, W, Ind, grad_output, dtype):
@@ -218,8 +242,8 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     dev = _require_gpu(X, W, Ind, grad_output)
     B, E, K, I, J = _check_shapes(X, W, Ind, grad_output, True)
     x_dtype, w_dtype = X.dtype, W.dtype
-    X, ld_b, ld_t = _rows_source(X.to(ct))
-    W = _dense16(W.to(ct)); Ind = Ind.contiguous(); grad_output = _dense16(grad_output.to(ct))
+    X, ld_b, ld_t = _rows_source(X, ct)
+    W = _dense16(W, ct); Ind = Ind.contiguous(); grad_output = _dense16(grad_output, ct)
     T = X.shape[1]
     grad_X = torch.empty((B, T, I), device=dev, dtype=ct)
     grad_W = torch.empty((E, I, J), device=dev, dtype=ct)
@@ -227,13 +251,14 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     mode = _MODES[_scatter_mode]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, (B, T, E, K, I, J), dt))
         rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
                                                    grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                    dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
     del keep
-    _abi.check(rc, "expert_gather_backward_call")
-    return grad_X.to(x_dtype), grad_W.to(w_dtype)
+    if rc:
+        _abi.check(rc, "expert_gather_backward_call")
+    return (grad_X if x_dtype is ct else grad_X.to(x_dtype)), (grad_W if w_dtype is ct else grad_W.to(w_dtype))
 
 
 def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
@@ -244,18 +269,19 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     if T < 0:
         raise ValueError("T must be non-negative")
     res_dtype = Y.dtype
-    Y = _dense16(Y.to(ct)); W = _dense16(W.to(ct)); Ind = Ind.contiguous()
+    Y = _dense16(Y, ct); W = _dense16(W, ct); Ind = Ind.contiguous()
     out = torch.empty((B, T, I), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
     mode = _MODES[_scatter_mode]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, mode, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, (B, T, E, K, I, J), dt))
         rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
                                                    ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
     del keep
-    _abi.check(rc, "expert_scatter_forward_call")
-    return out.to(res_dtype)
+    if rc:
+        _abi.check(rc, "expert_scatter_forward_call")
+    return out if res_dtype is ct else out.to(res_dtype)
 
 
 def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
@@ -263,21 +289,22 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
     dev = _require_gpu(Y, W, Ind, grad_X)
     B, E, K, I, J = _check_shapes(grad_X, W, Ind, Y, False)
     y_dtype, w_dtype = Y.dtype, W.dtype
-    grad_X, ld_b, ld_t = _rows_source(grad_X.to(ct))
-    Y = _dense16(Y.to(ct)); W = _dense16(W.to(ct)); Ind = Ind.contiguous()
+    grad_X, ld_b, ld_t = _rows_source(grad_X, ct)
+    Y = _dense16(Y, ct); W = _dense16(W, ct); Ind = Ind.contiguous()
     T = grad_X.shape[1]
     grad_Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     grad_W = torch.empty((E, J, I), device=dev, dtype=ct)
     d = _abi.Dims(B, T, E, K, I, J)
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _abi.lib().egs_workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, d, dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, (B, T, E, K, I, J), dt))
         rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
                                                     grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                     dt, _ind_type_id(Ind), _stream_ptr(dev))
     del keep
-    _abi.check(rc, "expert_scatter_backward_call")
-    return grad_Y.to(y_dtype), grad_W.to(w_dtype)
+    if rc:
+        _abi.check(rc, "expert_scatter_backward_call")
+    return (grad_Y if y_dtype is ct else grad_Y.to(y_dtype)), (grad_W if w_dtype is ct else grad_W.to(w_dtype))
 
 
 # module globals, bound by create_kernels() (reference egs/triton_kernels.py:26-29)
@@ -367,10 +394,38 @@ def create_kernels() -> None:
             return
         _register_ops(OP_NAMESPACE)
         ops = getattr(torch.ops, OP_NAMESPACE)
-        expert_gather_forward_call = ops.expert_gather_forward_call_fn
-        expert_gather_backward_call = ops.expert_gather_backward_call_fn
-        expert_scatter_forward_call = ops.expert_scatter_forward_call_fn
-        expert_scatter_backward_call = ops.expert_scatter_backward_call_fn
+        compiling = torch.compiler.is_compiling
+        plain = (torch.Tensor, torch.nn.Parameter)       # not a fake / functional / subclass tensor of some tracer
+
+        # The callables the Functions use.  Like the reference's (plain Python functions, egs/triton_kernels.py:569-578)
+        # they run the launcher directly for tensors on the GPU in eager mode, which saves the dispatcher's
+        # round trip per call (several microseconds, more than some of the kernels take); while torch.compile is
+        # tracing, and for meta / fake tensors, they go through the registered ops, whose fake implementations
+        # describe the outputs.
+        def gather_forward_call(X, W, Ind, out_dtype):
+            if type(X) in plain and X.is_cuda and not compiling():
+                return _gather_forward_impl(X, W, Ind, out_dtype)
+            return ops.expert_gather_forward_call_fn(X, W, Ind, out_dtype)
+
+        def gather_backward_call(X, W, Ind, grad_output, out_dtype):
+            if type(X) in plain and X.is_cuda and not compiling():
+                return _gather_backward_impl(X, W, Ind, grad_output, out_dtype)
+            return ops.expert_gather_backward_call_fn(X, W, Ind, grad_output, out_dtype)
+
+        def scatter_forward_call(Y, W, Ind, T, out_dtype):
+            if type(Y) in plain and Y.is_cuda and not compiling():
+                return _scatter_forward_impl(Y, W, Ind, T, out_dtype)
+            return ops.expert_scatter_forward_call_fn(Y, W, Ind, T, out_dtype)
+
+        def scatter_backward_call(Y, W, Ind, grad_X, out_dtype):
+            if type(Y) in plain and Y.is_cuda and not compiling():
+                return _scatter_backward_impl(Y, W, Ind, grad_X, out_dtype)
+            return ops.expert_scatter_backward_call_fn(Y, W, Ind, grad_X, out_dtype)
+
+        expert_gather_forward_call = gather_forward_call
+        expert_gather_backward_call = gather_backward_call
+        expert_scatter_forward_call = scatter_forward_call
+        expert_scatter_backward_call = scatter_backward_call
 
 
 def register_reference_namespace(ns: str = "mylib") -> None:
@@ -432,7 +487,7 @@ def expert_gather_fp8w_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.T
     B, E, K, I, J = _check_shapes(X, Wq, Ind, None, True)
     if tuple(scale.shape) != (E, J):
         raise ValueError(f"scale must be [E={E},J={J}], got {tuple(scale.shape)}")
-    X, ld_b, ld_t = _rows_source(X)
+    X, ld_b, ld_t = _rows_source(X, torch.bfloat16)
     Wq = Wq.contiguous(); scale = scale.contiguous(); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)
     d = _abi.Dims(B, X.shape[1], E, K, I, J)
@@ -458,7 +513,7 @@ def expert_gather_fp8_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.Te
     B, E, K, I, J = _check_shapes(X, Wq, Ind, None, True)
     if tuple(scale.shape) != (E, J):
         raise ValueError(f"scale must be [E={E},J={J}], got {tuple(scale.shape)}")
-    X, ld_b, ld_t = _rows_source(X)
+    X, ld_b, ld_t = _rows_source(X, torch.bfloat16)
     T = X.shape[1]
     Wq = Wq.contiguous(); scale = scale.contiguous(); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=X.dtype)

@@ -88,8 +88,10 @@ SMALL_SHAPES = [
 def force_generic(request):
     from expertscattergather_amd import _abi
     _abi.lib().egs_testing_force_generic(1 if request.param else 0)
+    hk._ws_sizes.clear()                    # remembered workspace sizes belong to the other kernel family
     yield request.param
     _abi.lib().egs_testing_force_generic(0)
+    hk._ws_sizes.clear()
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])

@@ -43,7 +43,9 @@ def test_ops_are_registered_with_fake_implementations():
     assert out.shape == (2, 5, 8)
     dY, dWs = ops.expert_scatter_backward_call_fn(Y, Ws, Ind, out, torch.float32)
     assert dY.shape == Y.shape and dWs.shape == Ws.shape
-    assert hk.expert_gather_forward_call is ops.expert_gather_forward_call_fn
+    # the module-level callables send meta tensors through the ops (and so through the fake implementations)
+    assert hk.expert_gather_forward_call(X, Wg, Ind, torch.float32).shape == (2, 4, 3, 6)
+    assert hk.expert_scatter_forward_call(Y, Ws, Ind, 5, torch.float32).shape == (2, 5, 8)
 
 
 def test_autograd_functions_trace_on_meta_tensors():
