@@ -7,6 +7,7 @@
 #include "egs_scatter_aux.h"
 #include "egs_small.h"
 #include "egs_dw_tile.h"
+#include "egs_small_f32.h"
 #include "egs_scatter_fused.h"
 
 #include <atomic>
@@ -373,6 +374,51 @@ int device_cu_count()
     return n;
 }
 
+// ---- fp32 gather of small experts (W(e) in LDS, fp32 matrix instruction)
+template <bool W_NMAJOR, int KS>
+int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t s)
+{
+    const size_t lds = rows_small_f32_lds(16 * KS, p.N);
+    switch (p.N / 16) {
+    case 1: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 1>), dim3(blocks), dim3(kThreads), lds, s, p); break;
+    case 2: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 2>), dim3(blocks), dim3(kThreads), lds, s, p); break;
+    case 3: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 3>), dim3(blocks), dim3(kThreads), lds, s, p); break;
+    default: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 4>), dim3(blocks), dim3(kThreads), lds, s, p); break;
+    }
+    EGS_CHECK_LAUNCH("rows_small_f32_kernel");
+    return EGS_OK;
+}
+
+// `used` reports whether the shape and operands qualified
+int gather_small_f32(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                     int ind_dtype, int w_layout, hipStream_t s, bool &used)
+{
+    used = false;
+    const int R = d->I, N = d->J;
+    if (g_force_generic || !(R == 32 || R == 64 || R == 128) || N % 16 != 0 || N < 16 || N > 64 || d->T == 0) return EGS_OK;
+    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16) || (ldx_b * 4) % 16 || (ldx_t * 4) % 16) return EGS_OK;
+    const int64_t Me = (int64_t)d->B * d->K;
+    if (Me == 0 || d->E == 0) return EGS_OK;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + R) * 4;
+    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 4 > kSpan32 || (uint64_t)Me * d->E * N * 4 > kSpan32) return EGS_OK;
+    SmallRowsParams p;
+    memset(&p, 0, sizeof(p));
+    p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y;
+    p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
+    p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
+    p.tiles_per_e = (int)((Me + 255) / 256);
+    if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return EGS_OK;
+    p.rows_share_xcd = 0;               // W(e) is fetched once per workgroup: experts share an XCD
+    const int blocks = 8 * ceil_div(p.E, 8) * p.tiles_per_e;
+    used = true;
+    const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
+    switch (R) {
+    case 32: return nmajor ? launch_gather_small_f32_ks<true, 2>(p, blocks, s) : launch_gather_small_f32_ks<false, 2>(p, blocks, s);
+    case 64: return nmajor ? launch_gather_small_f32_ks<true, 4>(p, blocks, s) : launch_gather_small_f32_ks<false, 4>(p, blocks, s);
+    default: return nmajor ? launch_gather_small_f32_ks<true, 8>(p, blocks, s) : launch_gather_small_f32_ks<false, 8>(p, blocks, s);
+    }
+}
+
 // ---- launch of a rows job, alone or sharing the launch with a weight gradient of the same call (its one-pass form,
 // or the first pass of its split form)
 template <class TT, bool W_NMAJOR, int KS, int TN, bool GATHER, bool OUT_F32>
@@ -669,6 +715,11 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
         SmallRowsJob j;
         if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j))
             return launch_rows_small_job(j, nullptr, nullptr, s);
+        if (act_dtype == EGS_F32 && w_dtype == EGS_F32) {
+            bool used = false;
+            const int rc = gather_small_f32(X, W, Ind, Y, d, ldx_b, ldx_t, ind_dtype, w_layout, s, used);
+            if (used) return rc;
+        }
     }
     RowsGemmParams p;
     memset(&p, 0, sizeof(p));
