@@ -81,6 +81,8 @@ SMALL_SHAPES = [
     (3, 64, 16, 16, 64, 56),      # J not a multiple of 16 (gather columns), scatter takes the general path
     (8, 60, 6, 20, 64, 128),      # reduction 128 on the one-kernel scatter, ragged 16-pick tiles
     (4, 300, 40, 25, 96, 32),     # 1000 picks per batch element, three 32-column slices
+    (2, 48, 40, 9, 72, 40),       # one-pass weight gradient with ragged 32 x 32 / 32 x 64 tiles (72 = 2 x 32 + 8, 40 = 32 + 8)
+    (1, 16, 64, 3, 40, 104),      # ... with fewer picks per expert (3) than one 32-pick step, many experts
 ]
 
 
