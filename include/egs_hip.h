@@ -45,7 +45,7 @@ typedef enum egs_status {
     EGS_ERR_BAD_DTYPE = -3,     /* counterpart of ValueError("Unknown dtype"), reference egs/triton_kernels.py:23 */
     EGS_ERR_BAD_LAYOUT = -4,
     EGS_ERR_BAD_MODE = -5,
-    EGS_ERR_WORKSPACE = -6,     /* workspace missing or smaller than egs_workspace_bytes() */
+    EGS_ERR_WORKSPACE = -6,     /* workspace missing, or smaller than the kernels selected for these operands need */
     EGS_ERR_ALIGNMENT = -7,
     EGS_ERR_HIP = -8,           /* a HIP runtime call failed; see egs_last_hip_error() */
     EGS_ERR_UNSUPPORTED = -9,
@@ -100,8 +100,12 @@ const char *egs_status_string(int status);
 /* text of the last HIP error seen by the calling thread ("" if none) */
 const char *egs_last_hip_error(void);
 
-/* bytes of scratch the op needs for these sizes (0 is a valid answer).
- * `mode` is an egs_scatter_mode and only matters for ops that scatter. */
+/* bytes of scratch the op needs for these sizes (0 is a valid answer: small experts in 16-bit types run on
+ * kernels that keep every intermediate on the CU).  `mode` is an egs_scatter_mode and only matters for ops
+ * that scatter.  The answer holds for dense operands that start on a 16-byte boundary (what hipMalloc and
+ * torch return); every entry point derives the requirement again from the operands it is given, and an
+ * operand off that grid can select a general kernel that needs more: the call then returns
+ * EGS_ERR_WORKSPACE and launches nothing; copy such operands to aligned storage first. */
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype);
 
 /* ---------------------------------------------------------------------------------------
