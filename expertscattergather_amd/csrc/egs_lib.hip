@@ -360,20 +360,6 @@ int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
     return EGS_OK;
 }
 
-// number of CUs of the current device (looked up once per device)
-int device_cu_count()
-{
-    static std::atomic<int> cached[kMaxDevices];
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
-    int n = cached[dev].load(std::memory_order_relaxed);
-    if (n == 0) {
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        cached[dev].store(n, std::memory_order_relaxed);
-    }
-    return n;
-}
-
 // ---- fp32 gather of small experts (W(e) in LDS, fp32 matrix instruction)
 template <bool W_NMAJOR, int KS>
 int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t s)
@@ -588,9 +574,15 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
 template <class TT, bool W_NMAJOR, int KS>
 int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
 {
-    static LdsGrant told_plain, told_dw, told_dwt;      // one set per template instantiation
+    static LdsGrant told_plain, told_dw, told_dwt, told_multi;      // one set per template instantiation
     if constexpr (TT::ES != 2) { dw = nullptr; dwt = nullptr; }     // the small weight gradients exist for 16-bit types only
-    if (dwt != nullptr) {
+    if (p.experts_per_pass < p.E) {
+        // several passes over groups of experts: a launch of its own (a weight gradient of the same call follows alone)
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_multi_kernel<TT, W_NMAJOR, KS>, told_multi, lds,
+                                           "hipFuncSetAttribute(scatter_fused_multi_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
+        hipLaunchKernelGGL((scatter_fused_multi_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
+    } else if (dwt != nullptr) {
       if constexpr (TT::ES == 2) {
         const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
         const size_t need = lds > tile_lds ? lds : tile_lds;
@@ -632,20 +624,40 @@ int launch_scatter_fused_ks(const ScatterFusedParams &p, int R, size_t lds, int 
     }
 }
 
-// Does the one-kernel scatter of small experts (product rows stay in LDS, no workspace) take this problem?
-bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype)
+// Does the one-kernel scatter of small experts (product rows stay in LDS, no workspace) take this problem, and in how
+// many passes over groups of experts?  experts_per_pass == E: one pass.
+struct FusedPlan { bool ok; int experts_per_pass; size_t lds; };
+
+FusedPlan scatter_fused_plan(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype)
 {
+    const FusedPlan no = {false, 0, 0};
     const int R = d->J, N = d->I;
     const int64_t NP = (int64_t)d->E * d->K;
-    if (g_force_generic || !(R == 32 || R == 64 || (R == 128 && act_dtype != EGS_F32))) return false;
+    if (g_force_generic || !(R == 32 || R == 64 || (R == 128 && act_dtype != EGS_F32))) return no;
     const int ES = elem_size(act_dtype);
-    if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 1024 || d->T < 1 || d->B < 1) return false;
-    if (scatter_fused_lds(d->T, (int)NP) > 156 * 1024) return false;
-    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 16)) return false;
-    if ((uint64_t)d->B * NP * R * ES > kSpan32 || (uint64_t)d->E * R * N * ES > kSpan32) return false;
+    if (N < kFusedCols || N % kFusedCols != 0 || NP < 1 || NP > 4096 || d->T < 1 || d->B < 1) return no;
+    if (!aligned_to(Y, 16) || !aligned_to(W, 16) || !aligned_to(Out, 16)) return no;
+    if ((uint64_t)d->B * NP * R * ES > kSpan32 || (uint64_t)d->E * R * N * ES > kSpan32) return no;
     const int slices = N / kFusedCols;
     const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
-    return blocks <= INT32_MAX / 2 && (int64_t)d->B * slices >= 8;      // fewer workgroups are not worth it
+    if (blocks > INT32_MAX / 2 || (int64_t)d->B * slices < 8) return no;        // fewer workgroups are not worth it
+    const size_t budget = 156 * 1024;
+    if (NP <= 1024 && scatter_fused_lds(d->T, (int)NP) <= budget) return {true, d->E, scatter_fused_lds(d->T, (int)NP)};
+    // groups of experts: as few passes as the rows' share of LDS allows, of equal size
+    if (d->T > (kFusedThreads >> 3) * kFusedMultiTokens) return no;
+    const size_t fixed = scatter_fused_lds(d->T, (int)NP, 0);
+    if (fixed >= budget) return no;
+    const int64_t fit = (int64_t)((budget - fixed) / ((size_t)d->K * kFusedCols * 4));     // experts whose rows fit
+    if (fit < 1) return no;
+    const int passes = ceil_div(d->E, (int)(fit < d->E ? fit : d->E));
+    if (passes < 2 || passes > kFusedMaxPasses) return no;
+    const int per_pass = ceil_div(d->E, passes);
+    return {true, per_pass, scatter_fused_lds(d->T, (int)NP, per_pass * d->K)};
+}
+
+bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype)
+{
+    return scatter_fused_plan(Y, W, Out, d, act_dtype).ok;
 }
 
 // GEMM-scatter of small experts in one kernel; the caller has checked scatter_fused_takes().  Both scatter modes
@@ -655,7 +667,9 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
 {
     const int R = d->J, N = d->I;
     const int64_t NP = (int64_t)d->E * d->K;
-    const size_t lds = scatter_fused_lds(d->T, (int)NP);
+    const FusedPlan fp = scatter_fused_plan(Y, W, Out, d, act_dtype);
+    if (!fp.ok) return EGS_ERR_UNSUPPORTED;
+    const size_t lds = fp.lds;
     const int slices = N / kFusedCols;
     const int64_t blocks = (int64_t)8 * ceil_div(d->B, 8) * slices;
     ScatterFusedParams p;
@@ -664,7 +678,8 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.B = d->B; p.T = d->T; p.E = d->E; p.K = d->K; p.N = N;
     p.ind_dtype = ind_dtype;
     p.slices = slices;
-    p.perm_at = (int32_t)(NP * kFusedCols * 4);
+    p.experts_per_pass = fp.experts_per_pass;
+    p.perm_at = (int32_t)((int64_t)fp.experts_per_pass * d->K * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
     if (act_dtype == EGS_F32)
@@ -1130,14 +1145,17 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
     DwTileJob dwt;
     if (g_small && w_elems > 0 &&
         make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt, /*wide=*/true)) {
-        // one launch, every workgroup on a CU of its own: the gather regridded to 8 wavefronts per workgroup
+        // One launch: the gather regridded to 8 wavefronts per workgroup, the weight-gradient workgroups first in launch
+        // order (they run longest).  The launch's LDS size admits one workgroup per CU, so the two bodies never share a
+        // CU (sharing one costs the sum of their times); with more workgroups than CUs the gather's fill the CUs the
+        // weight gradient leaves and then follow on each CU as it frees (B64 T256 E48 K32 I128 J64: 26.5 -> 21.1 us
+        // against two launches, B128 E32: 30.9 -> 21.3 us).
         SmallRowsJob g8 = gj;
         const int64_t Me = (int64_t)d->B * d->K;
         g8.p.tiles_per_e = (int)((Me + 511) / 512);
         if (g8.p.tiles_per_e % 8 != 0) g8.p.rows_share_xcd = 0;     // row tiles map to XCDs in groups of 8 only
         g8.blocks = g8.p.rows_share_xcd ? 8 * ceil_div(g8.p.tiles_per_e, 8) * g8.p.E : 8 * ceil_div(g8.p.E, 8) * g8.p.tiles_per_e;
-        const int cus = device_cu_count();
-        if (cus > 0 && g8.blocks + dwt.blocks <= cus) return launch_rows_small_job(g8, nullptr, &dwt, s);
+        if ((int64_t)g8.blocks + dwt.blocks <= INT32_MAX / 2) return launch_rows_small_job(g8, nullptr, &dwt, s);
     }
     const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt);
     if (dw_tile) {

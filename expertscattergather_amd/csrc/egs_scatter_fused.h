@@ -19,6 +19,11 @@
 // histograms fit in LDS; 16-bit elements with reduction 32/64/128 or fp32 with reduction 32/64, output
 // columns a multiple of 32.
 //
+// More picks than fit (MULTI, up to four passes): the table is in expert order inside a token's segment, so the
+// experts are taken in consecutive groups; each pass parks the products of one group in LDS and every thread
+// continues its tokens' sums where the previous pass stopped (a cursor per token, partial sums in
+// registers).  The order of the additions is the order of the table, as in one pass: same bits.
+//
 // Replaces the reference's expert_scatter_kernel (egs/triton_kernels.py:156-247), which adds every
 // output element with a global atomic.
 #pragma once
@@ -40,15 +45,21 @@ struct ScatterFusedParams {
     int32_t ind_dtype;
     int32_t slices;         // N / kFusedCols
     int32_t perm_at, cnt_at;    // byte offsets of the table and of the sort's counters in dynamic LDS (rows start at 0)
+    int32_t experts_per_pass;   // MULTI: experts whose product rows are in LDS at a time (E otherwise)
 };
 
-// LDS bytes: product rows, table, counters of the sort (one histogram per wavefront + offsets)
-__host__ __device__ inline size_t scatter_fused_lds(int T, int NP)
-{
-    return (size_t)NP * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)(kFusedThreads / 64 + 1) * T + 1) * 4 + 64;
-}
+constexpr int kFusedMaxPasses = 4;
+constexpr int kFusedMultiTokens = 8;    // MULTI: tokens per thread (64 threads groups of 8 walk the tokens) -> T <= 512
 
-template <class TT, bool W_NMAJOR, int KS>
+// LDS bytes: product rows (of `rows` picks at a time), table of all NP picks, counters of the sort (one histogram
+// per wavefront + offsets)
+__host__ __device__ inline size_t scatter_fused_lds(int T, int NP, int rows)
+{
+    return (size_t)rows * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)(kFusedThreads / 64 + 1) * T + 1) * 4 + 64;
+}
+__host__ __device__ inline size_t scatter_fused_lds(int T, int NP) { return scatter_fused_lds(T, NP, NP); }
+
+template <class TT, bool W_NMAJOR, int KS, bool MULTI = false>
 __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, const int block, char *smem)
 {
     // KS = reduction length in MFMA steps of four 16-byte chunks: 32 elements of a 16-bit type, 16 of fp32
@@ -75,14 +86,14 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 
     // ---------------- (1) units of work of this wavefront: (expert, pair of 16-pick row tiles); the weight
     // fragments of a unit serve both row tiles
+    // A pass covers the experts [e0, e0 + ne): all of them, unless MULTI
     const int KT2 = (K + 31) >> 5;
-    const int units = E * KT2;
     struct Unit { u32x4 y[2][KS]; u32x4 w[2 * KS]; };
     Unit buf[kFusedDepth];
     const uint32_t a_base_b = (uint32_t)b * (uint32_t)NP * R * ES;
-    auto load_unit = [&](Unit &u, int unit) {
-        if (unit >= units) return;                      // uniform per wavefront; a unit's own loads are unconditional
-        const int e = unit / KT2, rp = unit - e * KT2;
+    auto load_unit = [&](Unit &u, int unit, int e0, int ne) {
+        if (unit >= ne * KT2) return;                   // uniform per wavefront; a unit's own loads are unconditional
+        const int el = unit / KT2, rp = unit - el * KT2, e = e0 + el;
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             // coalesced: lanes 4r .. 4r+3 fetch four consecutive chunks of row r; transposed to operand order at use
@@ -119,9 +130,9 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
             }
         }
     };
-    auto compute_unit = [&](const Unit &u, int unit) {
-        if (unit >= units) return;
-        const int e = unit / KT2, rp = unit - e * KT2;
+    auto compute_unit = [&](const Unit &u, int unit, int ne) {
+        if (unit >= ne * KT2) return;
+        const int e = unit / KT2, rp = unit - e * KT2;  // expert counted from the first of the pass: rows are local to the pass
         f32x4 acc[2][2];
 #pragma unroll
         for (int h = 0; h < 2; ++h) { acc[h][0] = f32x4{0.f, 0.f, 0.f, 0.f}; acc[h][1] = f32x4{0.f, 0.f, 0.f, 0.f}; }
@@ -173,36 +184,14 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 
     // ---------------- (0) routing table of batch element b in LDS; the first units' operands go in flight
     // right behind the sort's token loads and travel while it runs
+    const int EP = MULTI ? p.experts_per_pass : E;
     csr_count_body(cnt, b, 0, tid, kFusedThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr, [&]() {
 #pragma unroll
-        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d);
+        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
     });
 
-    for (int u0 = wave; u0 < units; u0 += NWV * kFusedDepth) {
-#pragma unroll
-        for (int d = 0; d < kFusedDepth; ++d) {
-            compute_unit(buf[d], u0 + NWV * d);
-            load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth);
-        }
-    }
-    __syncthreads();
-
-    // ---------------- (2) per token: add its product rows in table order; 8 threads x 4 columns per token
     const int cc = tid & 7;
-    for (int t = tid >> 3; t < T; t += kFusedThreads >> 3) {
-        const int s0 = seg[t], s1 = seg[t + 1];
-        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int s = s0; s < s1; s += 4) {
-            int q[4];
-            f32x4 v[4];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) q[x] = perm[min(s + x, s1 - 1)];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)q[x] * kFusedCols)[cc ^ (q[x] & 7)];
-#pragma unroll
-            for (int x = 0; x < 4; ++x)
-                if (s + x < s1) sum += v[x];
-        }
+    auto store_row = [&](int t, const f32x4 &sum) {
         char *dst = p.out + (((size_t)b * T + t) * N + c0 + cc * 4) * ES;
         if constexpr (ES == 4) {
             *reinterpret_cast<f32x4 *>(dst) = sum;
@@ -212,6 +201,93 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
             w[1] = pack2<TT>(sum[2], sum[3]);
             *reinterpret_cast<u32x2 *>(dst) = w;
         }
+    };
+
+    if constexpr (!MULTI) {
+        for (int u0 = wave; u0 < E * KT2; u0 += NWV * kFusedDepth) {
+#pragma unroll
+            for (int d = 0; d < kFusedDepth; ++d) {
+                compute_unit(buf[d], u0 + NWV * d, E);
+                load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth, 0, E);
+            }
+        }
+        __syncthreads();
+
+        // ---------------- (2) per token: add its product rows in table order; 8 threads x 4 columns per token
+        for (int t = tid >> 3; t < T; t += kFusedThreads >> 3) {
+            const int s0 = seg[t], s1 = seg[t + 1];
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            for (int s = s0; s < s1; s += 4) {
+                int q[4];
+                f32x4 v[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) q[x] = perm[min(s + x, s1 - 1)];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)q[x] * kFusedCols)[cc ^ (q[x] & 7)];
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    if (s + x < s1) sum += v[x];
+            }
+            store_row(t, sum);
+        }
+    } else {
+        // ---------------- (1) + (2) in passes over groups of EP experts.  A thread keeps, for each of its tokens, the
+        // place in the segment where the previous pass stopped and the sum so far.
+        constexpr int TOK = kFusedMultiTokens, TSTRIDE = kFusedThreads >> 3;
+        int cur[TOK], end[TOK];
+        f32x4 sum[TOK];
+        for (int e0 = 0; e0 < E; e0 += EP) {
+            const int ne = min(EP, E - e0), ne_next = min(EP, E - e0 - ne);
+            for (int u0 = wave; u0 < ne * KT2; u0 += NWV * kFusedDepth) {
+#pragma unroll
+                for (int d = 0; d < kFusedDepth; ++d) {
+                    compute_unit(buf[d], u0 + NWV * d, ne);
+                    load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth, e0, ne);
+                }
+            }
+            // the next group's first operands travel while this group's rows are added
+            if (ne_next > 0) {
+#pragma unroll
+                for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, e0 + ne, ne_next);
+            }
+            __syncthreads();                            // products (and, in the first pass, the table) are in LDS
+            if (e0 == 0) {
+#pragma unroll
+                for (int i = 0; i < TOK; ++i) {
+                    const int t = (tid >> 3) + i * TSTRIDE;
+                    cur[i] = t < T ? seg[t] : 0;
+                    end[i] = t < T ? seg[t + 1] : 0;
+                    sum[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+            const int lo = e0 * K, hi = (e0 + ne) * K;  // picks whose rows are in LDS now; a segment lists its picks in increasing order
+#pragma unroll
+            for (int i = 0; i < TOK; ++i) {
+                while (cur[i] < end[i]) {
+                    int q[4];
+                    f32x4 v[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) q[x] = perm[min(cur[i] + x, end[i] - 1)];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int ql = q[x] < hi ? q[x] - lo : 0;       // picks of later groups: any valid row, not added
+                        v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)ql * kFusedCols)[cc ^ (ql & 7)];
+                    }
+                    int n = 0;
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (cur[i] + x < end[i] && q[x] < hi) { sum[i] += v[x]; ++n; }
+                    cur[i] += n;
+                    if (n < 4) break;
+                }
+            }
+            if (ne_next > 0) __syncthreads();           // everybody is done with this group's rows
+        }
+#pragma unroll
+        for (int i = 0; i < TOK; ++i) {
+            const int t = (tid >> 3) + i * TSTRIDE;
+            if (t < T) store_row(t, sum[i]);
+        }
     }
 }
 
@@ -220,6 +296,14 @@ __global__ __launch_bounds__(kFusedThreads) void scatter_fused_kernel(ScatterFus
 {
     extern __shared__ __attribute__((aligned(16))) char smem_fused[];
     scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused);
+}
+
+// more picks per batch element than LDS holds product rows for: groups of experts, one after the other
+template <class TT, bool W_NMAJOR, int KS>
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_multi_kernel(ScatterFusedParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_fused_multi[];
+    scatter_fused_body<TT, W_NMAJOR, KS, true>(p, (int)blockIdx.x, smem_fused_multi);
 }
 
 // the same with the first pass of a small weight gradient of the same backward call in the launch:

@@ -116,8 +116,9 @@ def test_workspace_sizes_are_consistent(lib):
         assert wb(op, 0, d, _abi.BF16) == 0 and wb(op, 1, d, _abi.BF16) == 0
     # more picks per batch element than the one-kernel scatter holds: routing table + fp32 product rows (deterministic) or
     # rows in the element type (atomic mode with a 16-bit type); fewer experts than the one-pass weight gradient wants: splits
-    d = _abi.Dims(16, 256, 8, 256, 128, 64)
-    rows = 16 * 8 * 256 * 128
+    assert wb(_abi.OP_GEMM_SCATTER, 0, _abi.Dims(16, 256, 8, 256, 128, 64), _abi.BF16) == 0   # 2048 picks: two passes, still no scratch
+    d = _abi.Dims(16, 256, 8, 640, 128, 64)
+    rows = 16 * 8 * 640 * 128
     det, fast, dw = wb(_abi.OP_GEMM_SCATTER, 0, d, _abi.BF16), wb(_abi.OP_GEMM_SCATTER, 1, d, _abi.BF16), wb(_abi.OP_DW, 0, d, _abi.BF16)
     assert rows * 4 <= det <= rows * 4 * 1.1 and rows * 2 <= fast <= rows * 2 * 1.1 and dw > 0
     assert wb(_abi.OP_GATHER_BACKWARD, 0, d, _abi.BF16) == det + dw

@@ -83,6 +83,11 @@ SMALL_SHAPES = [
     (4, 300, 40, 25, 96, 32),     # 1000 picks per batch element, three 32-column slices
     (2, 48, 40, 9, 72, 40),       # one-pass weight gradient with ragged 32 x 32 / 32 x 64 tiles (72 = 2 x 32 + 8, 40 = 32 + 8)
     (1, 16, 64, 3, 40, 104),      # ... with fewer picks per expert (3) than one 32-pick step, many experts
+    # one-kernel scatter in passes over groups of experts (more picks per batch element than LDS holds product rows for)
+    (2, 256, 48, 32, 128, 64),    # 1536 picks: two passes of 24 experts
+    (4, 100, 20, 100, 64, 32),    # 2000 picks, K = 100 (ragged 32-pick units): two passes of 10 experts
+    (8, 500, 33, 64, 32, 64),     # 2112 picks, T near the limit of 512, uneven last group (11 + 11 + 11 / 17 + 16)
+    (8, 64, 64, 64, 32, 32),      # 4096 picks: four passes of 16 experts
 ]
 
 
@@ -163,6 +168,20 @@ def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
     del junk
 
 
+def test_multi_pass_scatter_is_bitwise_reproducible_with_hot_tokens():
+    # 1536 picks per batch element on 5 tokens: every segment spans both passes of the one-kernel scatter
+    B, T, E, K, I, J = 4, 64, 48, 32, 64, 32
+    case = make_case(21, B, T, E, K, I, J, torch.bfloat16)
+    case["Ind"] = torch.randint(0, 5, (B, E, K), generator=torch.Generator().manual_seed(2))
+    Y, Ws, Ind = dev(case["Y"]), dev(case["Ws"]), dev(case["Ind"])
+    hk.set_scatter_mode("deterministic")
+    first = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    for _ in range(3):
+        assert torch.equal(first, hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32))
+    assert_close(first, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].numpy(), T), torch.bfloat16, "hot tokens, two passes")
+    assert first[:, 5:].abs().max().item() == 0.0      # tokens nobody picked
+
+
 @pytest.mark.parametrize("shape,dtype", [((3, 40, 6, 100, 24, 16), torch.float32),      # small-expert rows, table built by the general sorter
                                          ((2, 64, 8, 64, 128, 64), torch.bfloat16),     # small-expert rows, table rides along
                                          ((2, 50, 4, 300, 30, 24), torch.float16),      # I not a multiple of 4: scalar columns
@@ -230,8 +249,10 @@ def test_scatter_output_does_not_depend_on_stale_memory(mode):
                                          ((2, 64, 8, 16, 128, 64), torch.bfloat16),
                                          # the same with enough experts for the one-pass weight gradient (its rejected picks
                                          # get a buffer offset outside the descriptor) and its shared launch with the gather
-                                         ((8, 64, 32, 16, 128, 64), torch.float16)],
-                         ids=["small-f32", "large-bf16", "small-experts-bf16", "one-pass-dw-f16"])
+                                         ((8, 64, 32, 16, 128, 64), torch.float16),
+                                         # one-kernel scatter in two passes: a rejected pick has no place in the table
+                                         ((4, 64, 48, 32, 64, 32), torch.bfloat16)],
+                         ids=["small-f32", "large-bf16", "small-experts-bf16", "one-pass-dw-f16", "two-pass-scatter-bf16"])
 def test_out_of_range_picks_contribute_nothing(shape, dtype):
     B, T, E, K, I, J = shape
     case = make_case(13, B, T, E, K, I, J, dtype)
