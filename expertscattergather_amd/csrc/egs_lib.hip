@@ -315,9 +315,10 @@ bool make_dw_tile(const void *Xs, const void *Ys, const void *Ind, void *dW, con
                   int act_dtype, int out_dtype, int ind_dtype, int dw_layout, DwTileJob &j, bool wide = false)
 {
     if (g_force_generic || act_dtype == EGS_F32) return false;
-    if (d->I % 8 || d->J % 8 || d->I < 8 || d->J < 8 || d->I > 128 || d->J > 128) return false;
+    if (d->I % 8 || d->J % 8 || d->I < 8 || d->J < 8 || d->I > 2048 || d->J > 128) return false;
     const int64_t Me = (int64_t)d->B * d->K;
     if (Me == 0 || d->E == 0 || d->T == 0) return false;
+    if (d->I > 128 && d->J > 64 && Me >= 256) return false;        // the 256-row tiles of the direct-to-LDS kernel do better there
     const int it = ceil_div(d->I, 32), jt = ceil_div(d->J, wide ? 64 : 32);
     if ((int64_t)d->E * it * jt < (wide ? 64 : 128)) return false;
     if (!aligned_to(Xs, 16) || !aligned_to(Ys, 16) || !aligned_to(dW, 16) || (ldx_b * 2) % 16 || (ldx_t * 2) % 16) return false;
@@ -337,6 +338,17 @@ bool make_dw_tile(const void *Xs, const void *Ys, const void *Ind, void *dW, con
     j.act_dtype = act_dtype;
     j.wide = wide;
     return true;
+}
+
+// Which tile a one-pass weight gradient launched on its own should use.  32 x 64 tiles fetch whole 128-byte lines on
+// the Ys side and send half the requests per pick; 32 x 32 tiles only win when they fill the device exactly once and the
+// reduction is short (the reference's default shape: 10.1 against 10.6 us; E48: 15.0 / 11.5, B160: 24.5 / 21.2,
+// I256: 16.3 / 12.5 us).
+bool dw_tile_wide_alone(const egs_dims *d)
+{
+    constexpr int64_t kCUs = 256;
+    const int64_t narrow_tiles = (int64_t)d->E * ceil_div(d->I, 32) * ceil_div(d->J, 32);
+    return d->J > 32 && (narrow_tiles > kCUs || (int64_t)d->B * d->K >= 4096);
 }
 
 int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
@@ -582,7 +594,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
                                            "hipFuncSetAttribute(scatter_fused_multi_kernel)");
         if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_multi_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
-    } else if (dwt != nullptr) {
+    } else if (dwt != nullptr && !dwt->wide) {
       if constexpr (TT::ES == 2) {
         const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
         const size_t need = lds > tile_lds ? lds : tile_lds;
@@ -878,7 +890,7 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
     switch (dw_choose(Xs, Ys, dW, d, ldx_b, ldx_t, act_dtype, pl).path) {
     case DW_TILE: {
         DwTileJob jt;
-        make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt);
+        make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt, dw_tile_wide_alone(d));
         return launch_dw_tile_alone(jt, s);
     }
     case DW_SMALL: {
@@ -1100,7 +1112,13 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     const DwPlan dpl = plan_dw(d, dtype);
     SmallDwJob dwj;
     DwTileJob dwt;
-    const bool dw_tile = w_elems > 0 && make_dw_tile(X, grad_Y, Ind, grad_W, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dwt);
+    // 32 x 32 tiles when they can share the launch of the one-kernel scatter (one pass) and come after it in one round of
+    // workgroups, else what suits a launch of its own (I = 256: 42.9 us sharing, 37 us as two launches with 32 x 64 tiles)
+    const FusedPlan fpl = scatter_fused_plan(grad_Y, W, grad_X, d, dtype);
+    const bool shares_launch = fpl.ok && fpl.experts_per_pass == d->E &&
+                               (int64_t)d->E * ceil_div(d->I, 32) * ceil_div(d->J, 32) <= 256;
+    const bool dw_tile = w_elems > 0 && make_dw_tile(X, grad_Y, Ind, grad_W, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dwt,
+                                                     !shares_launch && dw_tile_wide_alone(d));
     const bool dw_small = !dw_tile && w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype,
                                                                    ind_dtype, EGS_W_EIJ, dpl, dwj);
     rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr,
@@ -1157,7 +1175,8 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
         g8.blocks = g8.p.rows_share_xcd ? 8 * ceil_div(g8.p.tiles_per_e, 8) * g8.p.E : 8 * ceil_div(g8.p.E, 8) * g8.p.tiles_per_e;
         if ((int64_t)g8.blocks + dwt.blocks <= INT32_MAX / 2) return launch_rows_small_job(g8, nullptr, &dwt, s);
     }
-    const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt);
+    const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt,
+                                                     dw_tile_wide_alone(d));
     if (dw_tile) {
         if (y_elems > 0) {
             rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);
