@@ -22,6 +22,7 @@
 // Replaces the reference's expert_gather_scatter_dW_kernel (egs/triton_kernels.py:261-356), which reduces
 // over the batch only and adds the K partial tiles with atomics in the output type.
 #pragma once
+#include <type_traits>
 #include "egs_device.h"
 
 namespace egs {
@@ -39,11 +40,19 @@ struct DwTileParams {
     uint32_t x_bytes, y_bytes;
 };
 
-// picks whose rows a wavefront keeps in flight at a time (registers: 16 or 24 per 32-pick step)
-__host__ __device__ constexpr int dw_tile_chunk(int TJ) { return TJ == 32 ? 256 : 128; }
-// per wavefront: row-offset tables of two chunks (Xs and Ys side) + two staging tiles (Xs piece 2 KB, Ys piece TJ * 64 bytes)
-__host__ __device__ constexpr int dw_tile_lds_per_wave(int TJ) { return 2 * 2 * dw_tile_chunk(TJ) * 4 + 2 * (2048 + TJ * 64); }
-__host__ __device__ constexpr size_t dw_tile_lds(int waves, int TJ = 32) { return (size_t)waves * dw_tile_lds_per_wave(TJ); }
+// `ES` = bytes per element (2, or 4 for fp32, whose pieces are twice as long and whose fragments are read untransposed)
+// picks whose rows a wavefront keeps in flight at a time (registers: 16 or 24 per 32-pick step; 32 or 48 in fp32)
+__host__ __device__ constexpr int dw_tile_chunk(int TJ, int ES = 2) { return (TJ == 32 ? 256 : 128) / (ES / 2); }
+// byte strides of a pick's piece inside a staging tile.  16-bit: dense (the transpose reads are XOR-swizzled instead).
+// fp32: 48 or 80 floats, so that the four picks a 4-byte fragment read touches (16 lanes each) fall on different banks
+__host__ __device__ constexpr int dw_tile_xstride(int ES) { return ES == 2 ? 64 : 192; }
+__host__ __device__ constexpr int dw_tile_ystride(int TJ, int ES) { return ES == 2 ? TJ * 2 : (TJ == 32 ? 192 : 320); }
+// per wavefront: row-offset tables of two chunks (Xs and Ys side) + two staging tiles (32 picks of each side)
+__host__ __device__ constexpr int dw_tile_lds_per_wave(int TJ, int ES = 2)
+{
+    return 2 * 2 * dw_tile_chunk(TJ, ES) * 4 + 2 * 32 * (dw_tile_xstride(ES) + dw_tile_ystride(TJ, ES));
+}
+__host__ __device__ constexpr size_t dw_tile_lds(int waves, int TJ = 32, int ES = 2) { return (size_t)waves * dw_tile_lds_per_wave(TJ, ES); }
 
 __device__ __forceinline__ u32x4 buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff)
 {
@@ -56,14 +65,19 @@ __device__ __forceinline__ u32x4 buffer_load16(__amdgpu_buffer_rsrc_t rsrc, uint
 template <class TT, int NW, int TJ = 32>
 __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int block, char *smem)
 {
-    static_assert(TT::ES == 2, "16-bit element types");
     static_assert(TJ == 32 || TJ == 64, "Ys-side tile width");
-    constexpr int CH = dw_tile_chunk(TJ), NS = CH / 32;
-    constexpr int kLdsPerWave = dw_tile_lds_per_wave(TJ);
-    constexpr int YB = TJ * 2;                  // bytes of a Ys piece
-    constexpr int YL = YB / 16;                 // lanes per Ys piece (4 or 8)
-    constexpr int YN = 32 * YL / 64;            // Ys loads per step (2 or 4), 64 / YL picks each
-    constexpr int STG = 2048 + 32 * YB;         // bytes of a staging tile
+    constexpr int ES = TT::ES;
+    constexpr int CH = dw_tile_chunk(TJ, ES), NS = CH / 32;
+    constexpr int kLdsPerWave = dw_tile_lds_per_wave(TJ, ES);
+    constexpr int XB = 32 * ES;                 // bytes of an Xs piece (32 columns)
+    constexpr int XL = XB / 16;                 // lanes per Xs piece (4; fp32: 8)
+    constexpr int XN = 32 * XL / 64;            // Xs loads per step (2; fp32: 4), 64 / XL picks each
+    constexpr int YB = TJ * ES;                 // bytes of a Ys piece
+    constexpr int YL = YB / 16;                 // lanes per Ys piece (4 or 8; fp32: 8 or 16)
+    constexpr int YN = 32 * YL / 64;            // Ys loads per step (2 or 4; fp32: 4 or 8), 64 / YL picks each
+    constexpr int XS = dw_tile_xstride(ES), YS = dw_tile_ystride(TJ, ES);
+    constexpr int XT = 32 * XS;                 // bytes of the Xs half of a staging tile
+    constexpr int STG = XT + 32 * YS;           // bytes of a staging tile
     constexpr int NY = TJ / 16;                 // 16-column groups on the Ys side
     int e, tile;
     const int tiles_per_e = p.i_tiles * p.j_tiles;
@@ -84,11 +98,11 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
     const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p.Xs), 0, (int)p.x_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_y = __builtin_amdgcn_make_buffer_rsrc(const_cast<char *>(p.Ys), 0, (int)p.y_bytes, 0x00020000);
 
-    // this lane's share of a step: Xs picks (lane >> 2) and 16 + (lane >> 2), 16-byte chunk (lane & 3) of the tile's
+    // this lane's share of a step: Xs picks (lane / XL) + (64 / XL) * h, 16-byte chunk lane % XL of the tile's
     // columns; Ys picks (lane / YL) + (64 / YL) * h, chunk lane % YL
-    const int xc = i0 + (lane & 3) * 8, yc = j0 + (lane % YL) * 8;
-    const uint32_t xcol = xc < p.I ? (uint32_t)xc * 2u : kVoffInvalid;
-    const uint32_t ycol = yc < p.J ? (uint32_t)yc * 2u : kVoffInvalid;
+    const int xc = i0 + (lane % XL) * (16 / ES), yc = j0 + (lane % YL) * (16 / ES);
+    const uint32_t xcol = xc < p.I ? (uint32_t)xc * (uint32_t)ES : kVoffInvalid;
+    const uint32_t ycol = yc < p.J ? (uint32_t)yc * (uint32_t)ES : kVoffInvalid;
 
     uint64_t iw[CH / 64];
     auto pick_of = [&](int c, int u, int &m, int &b) -> int64_t {
@@ -113,17 +127,17 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
             const int64_t pick = pick_of(c, u, m, b);
             const int64_t raw = decode_index_word(iw[u], p.Ind, p.ind_dtype, pick);
             const bool live = m < w_end && raw >= 0 && raw < (int64_t)p.T;
-            t[u * 64 + lane] = live ? (uint32_t)(((int64_t)b * p.ldx_b + raw * p.ldx_t) * 2) : kVoffInvalid;
-            t[CH + u * 64 + lane] = live ? (uint32_t)(pick * p.J * 2) : kVoffInvalid;
+            t[u * 64 + lane] = live ? (uint32_t)(((int64_t)b * p.ldx_b + raw * p.ldx_t) * ES) : kVoffInvalid;
+            t[CH + u * 64 + lane] = live ? (uint32_t)(pick * p.J * ES) : kVoffInvalid;
         }
     };
 
-    u32x4 rx[NS][2], ry[NS][YN];
+    u32x4 rx[NS][XN], ry[NS][YN];
     auto issue = [&](int c, int s) {
         const uint32_t *t = tab + (c & 1) * 2 * CH;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const uint32_t xo = t[s * 32 + h * 16 + (lane >> 2)];
+        for (int h = 0; h < XN; ++h) {
+            const uint32_t xo = t[s * 32 + h * (64 / XL) + lane / XL];
             rx[s][h] = buffer_load16(rs_x, (xo == kVoffInvalid || xcol == kVoffInvalid) ? kVoffInvalid : xo + xcol);
         }
 #pragma unroll
@@ -139,21 +153,24 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
 #pragma unroll
         for (int y = 0; y < NY; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // fragment addresses inside a piece ([32 picks][64 or YB bytes]): the lane points at pick 8 g + 4 h + a / 4 and the
-    // four columns 4 (a % 4) of a 16-column group, and receives column a of picks 8 g + 4 h .. + 3
+    // 16-bit fragment addresses inside a piece ([32 picks][64 or YB bytes]): the lane points at pick 8 g + 4 h + a / 4 and
+    // the four columns 4 (a % 4) of a 16-column group, and receives column a of picks 8 g + 4 h .. + 3
     // The 32-byte units of a row (one 16-column group each) are XOR-swizzled by the pick number so that the four picks
     // a transpose read touches per 16 lanes fall on different banks: unit ^ (pick / 2 % 2) in the 64-byte rows, unit ^
     // (pick % 4) in the 128-byte rows.  pick = 8 g + 4 h + a / 4 below, so the key depends on a / 4 only (and on h for
     // the 64-byte rows, where at1 = at0 + 4 rows keeps pick / 2 % 2).
+    // fp32 fragments are single elements: matrix-instruction step k of a 32-pick step takes pick 4 k + g from lane group g,
+    // column a of a 16-column group; rows are padded instead of swizzled (dw_tile_xstride).
     const int fr = a >> 2;                              // pick of the lane inside its group of four
     const int xkey = (fr >> 1) & 1, ykey = YB == 64 ? (fr >> 1) & 1 : fr & 3;
-    const int at0 = (g * 8 + fr) * 64 + (a & 3) * 8, at1 = at0 + 4 * 64;
-    const int yat0 = (g * 8 + fr) * YB + (a & 3) * 8, yat1 = yat0 + 4 * YB;
-    // writers: lane holds chunk c (16 bytes = half a unit) of pick p
-    const int xp = lane >> 2, xcn = lane & 3;
-    const int wr = xp * 64 + (((xcn >> 1) ^ ((xp >> 1) & 1)) << 5) + (xcn & 1) * 16;
+    const int at0 = ES == 2 ? (g * 8 + fr) * 64 + (a & 3) * 8 : g * XS + a * 4, at1 = at0 + 4 * 64;
+    const int yat0 = ES == 2 ? (g * 8 + fr) * YB + (a & 3) * 8 : g * YS + a * 4, yat1 = yat0 + 4 * YB;
+    // writers: lane holds chunk c (16 bytes; 16-bit: half a unit) of pick p
+    const int xp = lane / XL, xcn = lane % XL;
+    const int wr = ES == 2 ? xp * 64 + (((xcn >> 1) ^ ((xp >> 1) & 1)) << 5) + (xcn & 1) * 16 : xp * XS + xcn * 16;
     const int yp = lane / YL, ycn = lane % YL;
-    const int ywr = yp * YB + (((ycn >> 1) ^ (YB == 64 ? (yp >> 1) & 1 : yp & 3)) << 5) + (ycn & 1) * 16;
+    const int ywr = ES == 2 ? yp * YB + (((ycn >> 1) ^ (YB == 64 ? (yp >> 1) & 1 : yp & 3)) << 5) + (ycn & 1) * 16
+                            : yp * YS + ycn * 16;
     // A step goes registers -> LDS tile (stage_write), LDS tile -> fragments (stage_read), fragments -> MFMAs.  The
     // loop is software-pipelined: the fragments of step s are requested first, then the registers of step s+1 are
     // dropped into the other tile (and refilled from the next chunk), then the MFMAs of step s run - so the LDS
@@ -161,21 +178,37 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
     auto stage_write = [&](int s) {
         char *st = stage + (s & 1) * STG;
 #pragma unroll
-        for (int h = 0; h < 2; ++h) *reinterpret_cast<u32x4 *>(st + h * 1024 + wr) = rx[s][h];
+        for (int h = 0; h < XN; ++h) *reinterpret_cast<u32x4 *>(st + h * (64 / XL) * XS + wr) = rx[s][h];
 #pragma unroll
-        for (int h = 0; h < YN; ++h) *reinterpret_cast<u32x4 *>(st + 2048 + h * 1024 + ywr) = ry[s][h];
+        for (int h = 0; h < YN; ++h) *reinterpret_cast<u32x4 *>(st + XT + h * (64 / YL) * YS + ywr) = ry[s][h];
     };
-    auto stage_read = [&](int s, u32x4 (&pf)[2], u32x4 (&qf)[NY]) {
+    // fragments of a step: 16-bit, one 16-byte operand per 16-column group (8 picks per lane group);
+    // fp32, eight single elements per group (one per matrix-instruction step)
+    struct Frag16 { u32x4 v; };
+    struct Frag32 { float v[8]; };
+    typedef typename std::conditional<ES == 2, Frag16, Frag32>::type Frag;
+    auto stage_read = [&](int s, Frag (&pf)[2], Frag (&qf)[NY]) {
         const char *st = stage + (s & 1) * STG;
+        if constexpr (ES == 2) {
 #pragma unroll
-        for (int x = 0; x < 2; ++x) {
-            const u32x2 lo = lds_read_tr16(st + at0 + ((x ^ xkey) << 5)), hi = lds_read_tr16(st + at1 + ((x ^ xkey) << 5));
-            pf[x] = u32x4{lo[0], lo[1], hi[0], hi[1]};
-        }
+            for (int x = 0; x < 2; ++x) {
+                const u32x2 lo = lds_read_tr16(st + at0 + ((x ^ xkey) << 5)), hi = lds_read_tr16(st + at1 + ((x ^ xkey) << 5));
+                pf[x].v = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
 #pragma unroll
-        for (int y = 0; y < NY; ++y) {
-            const u32x2 lo = lds_read_tr16(st + 2048 + yat0 + ((y ^ ykey) << 5)), hi = lds_read_tr16(st + 2048 + yat1 + ((y ^ ykey) << 5));
-            qf[y] = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            for (int y = 0; y < NY; ++y) {
+                const u32x2 lo = lds_read_tr16(st + XT + yat0 + ((y ^ ykey) << 5)), hi = lds_read_tr16(st + XT + yat1 + ((y ^ ykey) << 5));
+                qf[y].v = u32x4{lo[0], lo[1], hi[0], hi[1]};
+            }
+        } else {
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) pf[x].v[k] = *reinterpret_cast<const float *>(st + at0 + k * 4 * XS + x * 64);
+#pragma unroll
+            for (int y = 0; y < NY; ++y)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) qf[y].v[k] = *reinterpret_cast<const float *>(st + XT + yat0 + k * 4 * YS + y * 64);
         }
     };
     auto chunk_len = [&](int c) { return c < nchunks ? min(CH, w_end - w_begin - c * CH) : 0; };
@@ -202,7 +235,7 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
             if (s * 32 < len) {
-                u32x4 pf[2], qf[NY];
+                Frag pf[2], qf[NY];
                 stage_read(s, pf, qf);
                 __builtin_amdgcn_sched_barrier(0);
                 if (s + 1 < NS && (s + 1) * 32 < len) {
@@ -213,10 +246,21 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
                     if (len2 > 0) issue(c + 2, 0);
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                if constexpr (ES == 2) {
 #pragma unroll
-                for (int x = 0; x < 2; ++x)
+                    for (int x = 0; x < 2; ++x)
 #pragma unroll
-                    for (int y = 0; y < NY; ++y) mma_chunk<TT>(acc[x][y], qf[y], pf[x]);
+                        for (int y = 0; y < NY; ++y) mma_chunk<TT>(acc[x][y], qf[y].v, pf[x].v);
+                } else {
+                    // accumulators interleaved: consecutive matrix instructions never wait for each other's result
+#pragma unroll
+                    for (int k = 0; k < 8; ++k)
+#pragma unroll
+                        for (int x = 0; x < 2; ++x)
+#pragma unroll
+                            for (int y = 0; y < NY; ++y)
+                                acc[x][y] = __builtin_amdgcn_mfma_f32_16x16x4f32(qf[y].v[k], pf[x].v[k], acc[x][y], 0, 0, 0);
+                }
             }
         }
     }
@@ -274,6 +318,13 @@ __global__ __launch_bounds__(kThreads) void dw_tile_kernel(DwTileParams p)
 {
     extern __shared__ __attribute__((aligned(16))) char smem_dw_tile[];
     dw_tile_body<TT, kThreads / 64>(p, (int)blockIdx.x, smem_dw_tile);
+}
+
+// fp32: 32 x 64 tiles, 4 wavefronts (the staging tiles of 8 would not fit)
+static __global__ __launch_bounds__(kThreads) void dw_tile_wide_f32_kernel(DwTileParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_dw_tile_wide_f32[];
+    dw_tile_body<ElemF32, kThreads / 64, 64>(p, (int)blockIdx.x, smem_dw_tile_wide_f32);
 }
 
 // 32 x 64 tiles, 8 wavefronts

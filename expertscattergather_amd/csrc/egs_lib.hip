@@ -314,16 +314,17 @@ bool make_dw_small(const void *Xs, const void *Ys, const void *Ind, void *dW, vo
 bool make_dw_tile(const void *Xs, const void *Ys, const void *Ind, void *dW, const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
                   int act_dtype, int out_dtype, int ind_dtype, int dw_layout, DwTileJob &j, bool wide = false)
 {
-    if (g_force_generic || act_dtype == EGS_F32) return false;
+    if (g_force_generic) return false;
+    const int ES = elem_size(act_dtype);
     if (d->I % 8 || d->J % 8 || d->I < 8 || d->J < 8 || d->I > 2048 || d->J > 128) return false;
     const int64_t Me = (int64_t)d->B * d->K;
     if (Me == 0 || d->E == 0 || d->T == 0) return false;
-    if (d->I > 128 && d->J > 64 && Me >= 256) return false;        // the 256-row tiles of the direct-to-LDS kernel do better there
+    if (ES == 2 && d->I > 128 && d->J > 64 && Me >= 256) return false;      // the 256-row tiles of the direct-to-LDS kernel do better there
     const int it = ceil_div(d->I, 32), jt = ceil_div(d->J, wide ? 64 : 32);
     if ((int64_t)d->E * it * jt < (wide ? 64 : 128)) return false;
-    if (!aligned_to(Xs, 16) || !aligned_to(Ys, 16) || !aligned_to(dW, 16) || (ldx_b * 2) % 16 || (ldx_t * 2) % 16) return false;
-    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * 2;
-    const uint64_t y_span = (uint64_t)Me * d->E * d->J * 2;
+    if (!aligned_to(Xs, 16) || !aligned_to(Ys, 16) || !aligned_to(dW, 16) || (ldx_b * ES) % 16 || (ldx_t * ES) % 16) return false;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + d->I) * ES;
+    const uint64_t y_span = (uint64_t)Me * d->E * d->J * ES;
     if (x_span >= (1ull << 31) || y_span >= (1ull << 31)) return false;
     if ((int64_t)8 * ceil_div(d->E, 8) * it * jt > INT32_MAX / 2) return false;
     memset(&j, 0, sizeof(j));
@@ -342,18 +343,31 @@ bool make_dw_tile(const void *Xs, const void *Ys, const void *Ind, void *dW, con
 
 // Which tile a one-pass weight gradient launched on its own should use.  32 x 64 tiles fetch whole 128-byte lines on
 // the Ys side and send half the requests per pick; 32 x 32 tiles only win when they fill the device exactly once and the
-// reduction is short (the reference's default shape: 10.1 against 10.6 us; E48: 15.0 / 11.5, B160: 24.5 / 21.2,
+// reduction is short (16-bit, the reference's default shape: 10.1 against 10.6 us; E48: 15.0 / 11.5, B160: 24.5 / 21.2,
 // I256: 16.3 / 12.5 us).
-bool dw_tile_wide_alone(const egs_dims *d)
+// In fp32 a wide tile is twice the matrix instructions for the same four wavefronts, so only the tile count decides
+// (default shape 19.5 / 30.1 us, B160: 41.7 / 67.3, E48: 36.2 / 30.5, I256: 36.6 / 31.0 us).
+bool dw_tile_wide_alone(const egs_dims *d, int act_dtype)
 {
     constexpr int64_t kCUs = 256;
     const int64_t narrow_tiles = (int64_t)d->E * ceil_div(d->I, 32) * ceil_div(d->J, 32);
-    return d->J > 32 && (narrow_tiles > kCUs || (int64_t)d->B * d->K >= 4096);
+    if (d->J <= 32) return false;
+    return narrow_tiles > kCUs || (act_dtype != EGS_F32 && (int64_t)d->B * d->K >= 4096);
 }
 
 int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
 {
-    if (j.wide) {
+    if (j.act_dtype == EGS_F32) {
+        // four wavefronts either way; both sizes of staging tiles need more than the default LDS limit
+        static LdsGrant told_narrow, told_wide;
+        const size_t lds = dw_tile_lds(kThreads / 64, j.wide ? 64 : 32, 4);
+        const int rc = j.wide
+            ? allow_large_lds((const void *)dw_tile_wide_f32_kernel, told_wide, lds, "hipFuncSetAttribute(dw_tile_wide_f32_kernel)")
+            : allow_large_lds((const void *)dw_tile_kernel<ElemF32>, told_narrow, lds, "hipFuncSetAttribute(dw_tile_kernel)");
+        if (rc != EGS_OK) return rc;
+        if (j.wide) hipLaunchKernelGGL(dw_tile_wide_f32_kernel, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
+        else hipLaunchKernelGGL(dw_tile_kernel<ElemF32>, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
+    } else if (j.wide) {
         static LdsGrant told_bf16, told_f16;
         const size_t lds = dw_tile_lds(kDwWideThreads / 64, 64);
         const int rc = j.act_dtype == EGS_BF16
@@ -890,7 +904,7 @@ int dw_impl(const void *Xs, const void *Ys, const void *Ind, void *dW, void *wor
     switch (dw_choose(Xs, Ys, dW, d, ldx_b, ldx_t, act_dtype, pl).path) {
     case DW_TILE: {
         DwTileJob jt;
-        make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt, dw_tile_wide_alone(d));
+        make_dw_tile(Xs, Ys, Ind, dW, d, ldx_b, ldx_t, act_dtype, out_dtype, ind_dtype, dw_layout, jt, dw_tile_wide_alone(d, act_dtype));
         return launch_dw_tile_alone(jt, s);
     }
     case DW_SMALL: {
@@ -1115,10 +1129,10 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     // 32 x 32 tiles when they can share the launch of the one-kernel scatter (one pass) and come after it in one round of
     // workgroups, else what suits a launch of its own (I = 256: 42.9 us sharing, 37 us as two launches with 32 x 64 tiles)
     const FusedPlan fpl = scatter_fused_plan(grad_Y, W, grad_X, d, dtype);
-    const bool shares_launch = fpl.ok && fpl.experts_per_pass == d->E &&
+    const bool shares_launch = dtype != EGS_F32 && fpl.ok && fpl.experts_per_pass == d->E &&
                                (int64_t)d->E * ceil_div(d->I, 32) * ceil_div(d->J, 32) <= 256;
     const bool dw_tile = w_elems > 0 && make_dw_tile(X, grad_Y, Ind, grad_W, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dwt,
-                                                     !shares_launch && dw_tile_wide_alone(d));
+                                                     !shares_launch && dw_tile_wide_alone(d, dtype));
     const bool dw_small = !dw_tile && w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype,
                                                                    ind_dtype, EGS_W_EIJ, dpl, dwj);
     rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr,
@@ -1176,7 +1190,7 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
         if ((int64_t)g8.blocks + dwt.blocks <= INT32_MAX / 2) return launch_rows_small_job(g8, nullptr, &dwt, s);
     }
     const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt,
-                                                     dw_tile_wide_alone(d));
+                                                     dw_tile_wide_alone(d, dtype));
     if (dw_tile) {
         if (y_elems > 0) {
             rc = gather_gemm_impl(grad_Out, W, Ind, grad_Y, nullptr, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);

@@ -250,9 +250,10 @@ def test_scatter_output_does_not_depend_on_stale_memory(mode):
                                          # the same with enough experts for the one-pass weight gradient (its rejected picks
                                          # get a buffer offset outside the descriptor) and its shared launch with the gather
                                          ((8, 64, 32, 16, 128, 64), torch.float16),
+                                         ((8, 64, 32, 16, 128, 64), torch.float32),         # fp32 form of the same kernels
                                          # one-kernel scatter in two passes: a rejected pick has no place in the table
                                          ((4, 64, 48, 32, 64, 32), torch.bfloat16)],
-                         ids=["small-f32", "large-bf16", "small-experts-bf16", "one-pass-dw-f16", "two-pass-scatter-bf16"])
+                         ids=["small-f32", "large-bf16", "small-experts-bf16", "one-pass-dw-f16", "one-pass-dw-f32", "two-pass-scatter-bf16"])
 def test_out_of_range_picks_contribute_nothing(shape, dtype):
     B, T, E, K, I, J = shape
     case = make_case(13, B, T, E, K, I, J, dtype)
