@@ -387,15 +387,19 @@ int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
 }
 
 // ---- fp32 gather of small experts (W(e) in LDS, fp32 matrix instruction)
+// Two 16-pick row tiles per wavefront and eight wavefronts per workgroup: two wavefronts per SIMD, so that one's waits
+// (row transposition, LDS fragment reads) sit under the other's matrix instructions (default shape 18.4 -> 16.8 us against
+// four row tiles and four wavefronts)
 template <bool W_NMAJOR, int KS>
 int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t s)
 {
+    constexpr int TQ = 2, threads = 64 * (16 / TQ);
     const size_t lds = rows_small_f32_lds(16 * KS, p.N);
     switch (p.N / 16) {
-    case 1: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 1>), dim3(blocks), dim3(kThreads), lds, s, p); break;
-    case 2: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 2>), dim3(blocks), dim3(kThreads), lds, s, p); break;
-    case 3: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 3>), dim3(blocks), dim3(kThreads), lds, s, p); break;
-    default: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 4>), dim3(blocks), dim3(kThreads), lds, s, p); break;
+    case 1: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 1, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
+    case 2: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 2, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
+    case 3: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 3, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
+    default: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 4, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
     }
     EGS_CHECK_LAUNCH("rows_small_f32_kernel");
     return EGS_OK;

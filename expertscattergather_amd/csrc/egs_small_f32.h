@@ -4,9 +4,9 @@
 // The fp32 matrix instruction (16x16x4) is the roof here (AI 40 FLOP/B against a ridge of 20), so the kernel is
 // arranged to keep it fed: W(e) - 32 KB at the default shape, too much for registers next to 64 picks - is brought
 // into LDS once per workgroup in [column][reduction] order, so that a lane's four reduction-consecutive weights are
-// one 16-byte LDS read shared by the four row tiles of its wavefront; the gathered rows go global -> registers ->
+// one 16-byte LDS read shared by the row tiles of its wavefront; the gathered rows go global -> registers ->
 // operand order (coalesced 64-byte runs per row, then the 4 x 16 lane transposition) a few 16-deep slabs ahead of
-// the MFMAs.  One wavefront = 64 picks of one expert, as in the 16-bit kernel; one barrier (W(e) in place).
+// the MFMAs.  One wavefront = 32 (or 64) picks of one expert, a workgroup 256; one barrier (W(e) in place).
 //
 // Replaces the reference's expert_gather_kernel (egs/triton_kernels.py:49-143) on these shapes.
 #pragma once
@@ -18,10 +18,12 @@ __host__ __device__ constexpr size_t rows_small_f32_lds(int R, int N) { return (
 
 // Requirements (checked by the launcher): fp32, R == 16 * KS in {32, 64, 128}, N == 16 * TN <= 64, rows of A, W and C
 // 16-byte aligned, every tensor below 4 GiB.  W is [E,R,N] (W_NMAJOR) or [E,N,R].
-template <bool W_NMAJOR, int KS, int TN>
-__global__ __launch_bounds__(kThreads) void rows_small_f32_kernel(SmallRowsParams p)
+// TQ = 16-pick row tiles per wavefront (4, or 2 with twice the wavefronts: a workgroup covers 256 picks either way)
+template <bool W_NMAJOR, int KS, int TN, int TQ = 4>
+__global__ __launch_bounds__(64 * (16 / TQ)) void rows_small_f32_kernel(SmallRowsParams p)
 {
-    constexpr int TQ = 4, R = 16 * KS, N = 16 * TN, LDW = R + 4;        // LDW: padded so that the 16 lanes of a read spread over the banks
+    constexpr int R = 16 * KS, N = 16 * TN, LDW = R + 4;        // LDW: padded so that the 16 lanes of a read spread over the banks
+    constexpr int PW = 16 * TQ, NTHREADS = 64 * (256 / PW);     // picks per wavefront, threads per workgroup
     constexpr int PF = KS < 4 ? KS : 4;                                 // slabs of gathered rows in flight
     extern __shared__ __attribute__((aligned(16))) float w_lds[];      // [N][LDW]
     int e, tile;
@@ -31,31 +33,26 @@ __global__ __launch_bounds__(kThreads) void rows_small_f32_kernel(SmallRowsParam
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
-    const int m0 = (tile * 4 + wave) * 64;
+    const int m0 = (tile * (256 / PW) + wave) * PW;
     const bool live_wave = m0 < Me;
 
-    // the index load goes first: the chain index -> row is the long one
-    const int m_lane = m0 + lane;
+    // the index load goes first: the chain index -> row is the long one (lanes beyond the wavefront's picks repeat them
+    // and own nothing)
+    const int m_lane = m0 + lane % PW;
     const int mm_lane = min(m_lane, Me - 1);
     const int b_lane = mm_lane / p.K;
     const int64_t pick = ((int64_t)b_lane * p.E + e) * p.K + (mm_lane - b_lane * p.K);
     uint64_t t_word = 0;
     if (live_wave) t_word = load_index_word(p.Ind, p.ind_dtype, pick);
 
-    // W(e) -> LDS as [column][reduction]
+    // W(e) -> registers (all loads in flight behind the index load), LDS as [column][reduction] further down
     const char *We = p.W + (size_t)e * R * N * 4;
-    if constexpr (!W_NMAJOR) {          // stored [N][R]: rows copied as they are
-        for (int c = tid; c < N * (R / 4); c += kThreads) {
-            const int n = c / (R / 4), k4 = c - n * (R / 4);
-            *reinterpret_cast<u32x4 *>(w_lds + n * LDW + 4 * k4) = *reinterpret_cast<const u32x4 *>(We + ((size_t)n * R + 4 * k4) * 4);
-        }
-    } else {                            // stored [R][N]: four columns of one reduction row per thread, written transposed
-        for (int c = tid; c < R * (N / 4); c += kThreads) {
-            const int r = c / (N / 4), n4 = c - r * (N / 4);
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(We + ((size_t)r * N + 4 * n4) * 4);
+    constexpr int W_CHUNKS = R * N / 4, W_IT = (W_CHUNKS + NTHREADS - 1) / NTHREADS;
+    u32x4 wv[W_IT];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) w_lds[(4 * n4 + i) * LDW + r] = bits_f32(v[i]);
-        }
+    for (int i = 0; i < W_IT; ++i) {
+        const int c = min(tid + i * NTHREADS, W_CHUNKS - 1);
+        wv[i] = *reinterpret_cast<const u32x4 *>(We + (size_t)c * 16);      // both layouts are read as they lie
     }
 
     uint32_t aoff = 0, coff = 0;
@@ -65,7 +62,7 @@ __global__ __launch_bounds__(kThreads) void rows_small_f32_kernel(SmallRowsParam
         const int32_t t = (t_raw < 0 || t_raw >= (int64_t)p.T) ? -1 : (int32_t)t_raw;
         if (t >= 0) aoff = (uint32_t)(((int64_t)b_lane * p.lda_b + (int64_t)t * p.lda_t) * 4);
         coff = (uint32_t)(pick * N * 4);
-        state = m_lane < Me ? (t >= 0 ? 1 : 2) : 0;
+        state = (m_lane < Me && lane < PW) ? (t >= 0 ? 1 : 2) : 0;
     }
     // gathered rows: lanes 4r .. 4r+3 fetch the four 16-byte chunks of a 16-deep slab of row 16 tq + r
     uint32_t xo[TQ];
@@ -77,6 +74,20 @@ __global__ __launch_bounds__(kThreads) void rows_small_f32_kernel(SmallRowsParam
         for (int s = 0; s < PF; ++s)
 #pragma unroll
             for (int tq = 0; tq < TQ; ++tq) xr[s][tq] = *reinterpret_cast<const u32x4 *>(p.A + xo[tq] + s * 64);
+    }
+#pragma unroll
+    for (int i = 0; i < W_IT; ++i) {
+        const int c = tid + i * NTHREADS;
+        if (c < W_CHUNKS) {
+            if constexpr (!W_NMAJOR) {      // stored [N][R]: rows copied as they are
+                const int n = c / (R / 4), k4 = c - n * (R / 4);
+                *reinterpret_cast<u32x4 *>(w_lds + n * LDW + 4 * k4) = wv[i];
+            } else {                        // stored [R][N]: four columns of one reduction row per thread, written transposed
+                const int r = c / (N / 4), n4 = c - r * (N / 4);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) w_lds[(4 * n4 + x) * LDW + r] = bits_f32(wv[i][x]);
+            }
+        }
     }
     __syncthreads();                    // W(e) is in place
     if (!live_wave) return;
