@@ -23,6 +23,8 @@ IND_I16, IND_I32, IND_I64, IND_U8 = 0, 1, 2, 3
 W_EIJ, W_EJI = 0, 1
 SCATTER_DETERMINISTIC, SCATTER_ATOMIC = 0, 1
 OP_GATHER_GEMM, OP_GEMM_SCATTER, OP_DW, OP_GATHER_BACKWARD, OP_SCATTER_BACKWARD = 0, 1, 2, 3, 4
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU, ACT_GELU_TANH = 0, 1, 2, 3, 4
+EGS_ERR_UNSUPPORTED = -9
 ABI_VERSION = 1
 
 
@@ -51,6 +53,8 @@ SIGNATURES = {
     "egs_expert_scatter_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _vp]),
     "egs_expert_scatter_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _vp]),
     "egs_validate_indices": (_i, [_vp, _i, _i64, ctypes.c_int32, _vp, _vp]),
+    "egs_expert_mlp_supported": (_i, [_dp, _i]),
+    "egs_expert_mlp_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _vp]),
 }
 
 _lib = None

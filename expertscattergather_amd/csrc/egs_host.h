@@ -21,6 +21,13 @@ extern std::atomic<bool> g_force_generic;       // testing aid (egs_testing_forc
 int hip_fail(hipError_t err, const char *what);     // records the HIP error text for egs_last_hip_error, returns EGS_ERR_HIP
 const char *last_hip_error();
 
+// A kernel that takes more than 64 KB of dynamic LDS has to be granted it, per device.  One LdsGrant per kernel
+// (a function-local static at the launch site) remembers the largest size granted on each device; growth is
+// serialised so that a smaller request racing with a larger one cannot shrink the grant.
+constexpr int kMaxDevices = 64;
+struct LdsGrant { std::atomic<uint32_t> bytes[kMaxDevices]; };
+int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *what);
+
 #define EGS_CHECK_LAUNCH(what)                                         \
     do {                                                               \
         hipError_t err__ = hipGetLastError();                          \

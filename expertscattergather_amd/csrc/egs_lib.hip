@@ -29,28 +29,7 @@ int hip_fail(hipError_t err, const char *what)
 }
 const char *last_hip_error() { return g_hip_error_buf; }
 
-}  // namespace host
-}  // namespace egs
-
-namespace {
-
-// ------------------------------------------------------------------------------ built-in scratch
-// Device memory that exists from the moment the library's code object is loaded, for the one entry
-// point that serves callers which cannot allocate (egs_dw_builtin_scratch).  Every GPU the library
-// runs on holds its own copy of the array, at its own address, until the process ends.
-// The array's name is only a host-side handle: host code never passes it to a kernel or a copy.  The
-// device address is looked up once per device (with that device current) and kept.
-static __device__ __align__(256) unsigned char scratch[EGS_BUILTIN_SCRATCH_BYTES];
-
-constexpr int kMaxDevices = 64;
-std::mutex g_scratch_mutex;
-void *g_scratch_ptr[kMaxDevices];              // per device: address of that device's copy of `scratch`
-
-// A kernel that takes more than 64 KB of dynamic LDS has to be granted it, per device.  One LdsGrant per kernel
-// remembers the largest size granted on each device; growth is serialised so that a smaller request racing
-// with a larger one cannot shrink the grant.
-struct LdsGrant { std::atomic<uint32_t> bytes[kMaxDevices]; };
-std::mutex g_lds_mutex;
+static std::mutex g_lds_mutex;
 int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *what)
 {
     if (lds <= 64 * 1024) return EGS_OK;
@@ -66,6 +45,22 @@ int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *wha
     grant.bytes[dev].store((uint32_t)lds, std::memory_order_release);
     return EGS_OK;
 }
+
+}  // namespace host
+}  // namespace egs
+
+namespace {
+
+// ------------------------------------------------------------------------------ built-in scratch
+// Device memory that exists from the moment the library's code object is loaded, for the one entry
+// point that serves callers which cannot allocate (egs_dw_builtin_scratch).  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends.
+// The array's name is only a host-side handle: host code never passes it to a kernel or a copy.  The
+// device address is looked up once per device (with that device current) and kept.
+static __device__ __align__(256) unsigned char scratch[EGS_BUILTIN_SCRATCH_BYTES];
+
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];              // per device: address of that device's copy of `scratch`
 
 int builtin_scratch_ptr(void **out)
 {

@@ -26,7 +26,7 @@ from . import _abi
 __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
     "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
-    "register_reference_namespace", "release_workspaces",
+    "register_reference_namespace", "release_workspaces", "expert_mlp_forward",
 ]
 
 OP_NAMESPACE = "egs_amd"
@@ -531,6 +531,69 @@ def expert_gather_fp8_forward(X: torch.Tensor, Wq: torch.Tensor, scale: torch.Te
     Xq = ws[:B * T * I].view(torch.float8_e4m3fn).view(B, T, I)
     xs = ws[xq_bytes:xq_bytes + B * T * 4].view(torch.float32).view(B, T)
     return Y, Xq, xs
+
+
+_ACTIVATIONS = {None: _abi.ACT_NONE, "none": _abi.ACT_NONE, "identity": _abi.ACT_NONE, "relu": _abi.ACT_RELU,
+                "gelu": _abi.ACT_GELU, "silu": _abi.ACT_SILU, "swish": _abi.ACT_SILU, "gelu_tanh": _abi.ACT_GELU_TANH}
+_TORCH_ACT = {
+    _abi.ACT_NONE: lambda y: y,
+    _abi.ACT_RELU: torch.relu,
+    _abi.ACT_GELU: torch.nn.functional.gelu,
+    _abi.ACT_SILU: torch.nn.functional.silu,
+    _abi.ACT_GELU_TANH: lambda y: torch.nn.functional.gelu(y, approximate="tanh"),
+}
+
+
+def _mlp_block_pays(B: int, E: int, I: int, J: int, act: int) -> bool:
+    """Measured on MI355X (bf16): the one kernel wins while its workgroups fit one round of the device (256) and the
+    activation is cheap or the experts few; B64 T256 E32 K32 I128 J64: relu 22.8 against 27.3 us, gelu 33.1 against
+    28.9 us; E16: 14.6 / 23.3 us and 21.0 / 23.0 us; B128: 43.3 / 41.6 us."""
+    blocks = 8 * ((B + 7) // 8) * (I // 32)
+    cheap = act in (_abi.ACT_NONE, _abi.ACT_RELU)
+    return blocks <= 256 and (cheap or E * I * J <= 16 * 128 * 64)
+
+
+def expert_mlp_forward(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor,
+                       activation="relu", force_block: bool = False) -> torch.Tensor:
+    """Inference block ``scatter(act(gather(X, W_gather, Ind)), W_scatter, Ind, T)`` - the call pattern of the
+    reference's layers (test_speed.ipynb:73-75 on egs/triton_kernels.py:49-143, :156-247) - without autograd.
+
+    X [B,T,I], W_gather [E,I,J], W_scatter [E,J,I], Ind [B,E,K] -> [B,T,I].  For small experts in a 16-bit type
+    (I in {32, 64, 128}, J in {32, 64}, at most 1024 picks per batch element) this is ONE kernel and the rows
+    Y [B,E,K,J] between the two products never exist in memory; every other case, and every case where the one
+    kernel is known to lose (more workgroups than one round of the device, or an expensive activation on many
+    experts: its four slice workgroups per batch element each repeat the gather product), runs the two forward
+    launchers with torch's activation in between (on the GPU all the same).  ``force_block=True`` takes the one
+    kernel whenever it can run.  ``activation``: "none", "relu",
+    "gelu", "gelu_tanh", "silu".  The activation is applied to the fp32 product and rounded to the element
+    type once, exactly where a stored Y would have been rounded."""
+    if activation not in _ACTIVATIONS:
+        raise ValueError(f"activation must be one of {sorted(k for k in _ACTIVATIONS if k)}, got {activation!r}")
+    act = _ACTIVATIONS[activation]
+    dev = _require_gpu(X, W_gather, W_scatter, Ind)
+    B, E, K, I, J = _check_shapes(X, W_gather, Ind, None, True)
+    if W_scatter.dim() != 3 or tuple(W_scatter.shape) != (E, J, I):
+        raise ValueError(f"W_scatter must be [E,J,I] = {(E, J, I)}, got {tuple(W_scatter.shape)}")
+    ct = _compute_dtype(torch.float32, X, W_gather, W_scatter)
+    T = X.shape[1]
+    d = _abi.Dims(B, T, E, K, I, J)
+    lib = _abi.lib()
+    if ct is not torch.float32 and (force_block or _mlp_block_pays(B, E, I, J, act)) \
+            and lib.egs_expert_mlp_supported(d, dtype_to_type_id(ct)):
+        res_dtype = X.dtype
+        Xs, ld_b, ld_t = _rows_source(X, ct)
+        Wg = _dense16(W_gather, ct); Ws = _dense16(W_scatter, ct); Indc = Ind.contiguous()
+        out = torch.empty((B, T, I), device=dev, dtype=ct)
+        with _on_device(dev):
+            rc = lib.egs_expert_mlp_forward(Xs.data_ptr(), Wg.data_ptr(), Ws.data_ptr(), Indc.data_ptr(), out.data_ptr(), d,
+                                            ld_b, ld_t, dtype_to_type_id(ct), _ind_type_id(Indc), act, _stream_ptr(dev))
+        if rc == 0:
+            return out if res_dtype is ct else out.to(res_dtype)
+        if rc != _abi.EGS_ERR_UNSUPPORTED:
+            _abi.check(rc, "expert_mlp_forward")
+    with torch.no_grad():
+        Y = _TORCH_ACT[act](_gather_forward_impl(X, W_gather, Ind, torch.float32))
+        return _scatter_forward_impl(Y, W_scatter, Ind, T, torch.float32)
 
 
 def validate_indices(Ind: torch.Tensor, T: int) -> int:

@@ -176,6 +176,32 @@ int egs_gather_gemm_fp8act(const void *X, const void *Wq, const float *w_scale, 
                            int64_t ldx_b, int64_t ldx_t, int ind_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Inference block (new; no single kernel of the reference corresponds to it): the reference's call pattern
+ *   out = scatter(act(gather(x, Ind)), Ind, T)          (test_speed.ipynb:73-75)
+ * in ONE kernel for small experts; the rows Y[B,E,K,J] between the two products stay in registers:
+ *   Out[b,t,:] = sum over picks (e,k) of t, in pick order, of  act(X[b,Ind[b,e,k],:] . Wg[e]) . Ws[e]
+ * Wg is [E,I,J], Ws is [E,J,I], Out [B,T,I] is written completely (tokens nobody picked become zero); the
+ * activation is applied to the fp32 product and the result rounded to the element type, as a stored Y would
+ * be.  Bitwise reproducible, no workspace.  Taken for 16-bit types, I in {32, 64, 128}, J in {32, 64} and at most 1024
+ * picks per batch element (egs_expert_mlp_supported); anything else returns EGS_ERR_UNSUPPORTED and the caller composes
+ * egs_expert_gather_forward, its own activation and egs_expert_scatter_forward.
+ * ------------------------------------------------------------------------------------- */
+typedef enum egs_activation {
+    EGS_ACT_NONE = 0,
+    EGS_ACT_RELU = 1,
+    EGS_ACT_GELU = 2,           /* erf form (torch.nn.functional.gelu default) */
+    EGS_ACT_SILU = 3,
+    EGS_ACT_GELU_TANH = 4       /* tanh approximation */
+} egs_activation;
+
+/* 1 if egs_expert_mlp_forward takes these sizes (with dense operands that start on a 16-byte boundary), else 0 */
+int egs_expert_mlp_supported(const egs_dims *d, int dtype);
+
+int egs_expert_mlp_forward(const void *X, const void *Wg, const void *Ws, const void *Ind, void *Out,
+                           const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                           int dtype, int ind_dtype, int activation, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Launcher-level entry points (one per reference callable)
  * ------------------------------------------------------------------------------------- */
 

@@ -139,3 +139,22 @@ def test_check_raises_like_the_reference():
     with pytest.raises(RuntimeError, match="workspace"):
         _abi.check(-6, "x")
     _abi.check(0, "x")
+
+
+def test_inference_block_entry_point_validates_without_a_gpu(lib):
+    ok = _abi.Dims(64, 256, 32, 32, 128, 64)
+    assert lib.egs_expert_mlp_supported(ok, _abi.BF16) == 1 and lib.egs_expert_mlp_supported(ok, _abi.F16) == 1
+    assert lib.egs_expert_mlp_supported(ok, _abi.F32) == 0                                         # 16-bit types only
+    assert lib.egs_expert_mlp_supported(_abi.Dims(64, 256, 32, 32, 128, 128), _abi.BF16) == 0      # J = 128
+    assert lib.egs_expert_mlp_supported(_abi.Dims(64, 256, 32, 64, 128, 64), _abi.BF16) == 0       # 2048 picks per batch element
+    assert lib.egs_expert_mlp_supported(_abi.Dims(64, 256, 32, 32, 96, 64), _abi.BF16) == 0        # I not 32 / 64 / 128
+    p = 0x1000
+    args = (p, p, p, p, p)
+    assert lib.egs_expert_mlp_forward(*args, ok, 256 * 128, 128, _abi.BF16, _abi.IND_I64, 9, None) == -5    # unknown activation
+    assert lib.egs_expert_mlp_forward(*args, ok, 256 * 128, 128, 7, _abi.IND_I64, _abi.ACT_RELU, None) == _abi.EGS_ERR_BAD_DTYPE
+    assert lib.egs_expert_mlp_forward(*args, ok, 256 * 128, 64, _abi.BF16, _abi.IND_I64, _abi.ACT_RELU, None) == -10   # token stride < I
+    assert lib.egs_expert_mlp_forward(None, p, p, p, p, ok, 256 * 128, 128, _abi.BF16, _abi.IND_I64, _abi.ACT_RELU, None) == -1
+    assert lib.egs_expert_mlp_forward(*args, _abi.Dims(64, 256, 32, 32, 128, 128), 256 * 128, 128, _abi.BF16, _abi.IND_I64,
+                                      _abi.ACT_RELU, None) == _abi.EGS_ERR_UNSUPPORTED
+    assert lib.egs_expert_mlp_forward(p, p, p, p, p + 2, ok, 256 * 128, 128, _abi.BF16, _abi.IND_I64, _abi.ACT_RELU,
+                                      None) == _abi.EGS_ERR_UNSUPPORTED                                # output off the 16-byte grid

@@ -599,3 +599,97 @@ def test_modules_trace_through_torch_compile():
         assert torch.equal(a, b), f"{name}: compiled differs from eager"
     assert_close(eager[0], O.scatter_forward(np64(gather(dev(case["X"]), Ind)), np64(case["Ws"]), case["Ind"].numpy(), T),
                  torch.bfloat16, "compiled block")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# inference block: scatter(act(gather(x, Ind)), Ind, T) in one kernel (reference call pattern test_speed.ipynb:73-75)
+def _np_act(y, name):
+    from scipy.special import erf
+    if name == "relu":
+        return np.maximum(y, 0.0)
+    if name == "gelu":
+        return 0.5 * y * (1.0 + erf(y / np.sqrt(2.0)))
+    if name == "gelu_tanh":
+        return 0.5 * y * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (y + 0.044715 * y ** 3)))
+    if name == "silu":
+        return y / (1.0 + np.exp(-y))
+    return y
+
+
+def _mlp_oracle(case, T, act, dtype, stored_y=False):
+    """The oracle's gather, the activation in float64, one rounding to the element type where a stored Y would be
+    rounded, the oracle's scatter.  `stored_y`: Y is also rounded before the activation (separate launches)."""
+    X, Wg, Ws = (np64(case[k]) for k in ("X", "Wg", "Ws"))
+    Ind = case["Ind"].numpy()
+    bad = (Ind < 0) | (Ind >= T)
+    safe = np.where(bad, 0, Ind)
+    Y = O.gather_forward(X, Wg, safe)
+    if stored_y:
+        Y = np64(torch.from_numpy(Y).to(dtype))
+    Y = _np_act(Y, act) * (~bad)[..., None]
+    Y = np64(torch.from_numpy(Y).to(dtype))
+    return O.scatter_forward(Y, Ws, safe, T)
+
+
+MLP_SHAPES = [
+    (4, 64, 8, 16, 128, 64),      # default-like, scaled down
+    (2, 256, 32, 32, 128, 64),    # two batch elements of the default shape
+    (4, 50, 9, 11, 64, 32),       # J = 32: half of the lanes of the second product carry nothing; ragged K, E
+    (5, 40, 12, 33, 128, 64),     # K = 33: a second, nearly empty unit per expert
+    (8, 33, 5, 64, 32, 64),       # I = 32: one output slice, one step of the first product
+    (4, 700, 8, 20, 64, 32),      # long T
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("shape", MLP_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_inference_block_matches_oracle(shape, dtype):
+    from expertscattergather_amd import _abi
+    B, T, E, K, I, J = shape
+    assert _abi.lib().egs_expert_mlp_supported(_abi.Dims(*shape), hk.dtype_to_type_id(dtype)) == 1
+    case = make_case(31, B, T, E, K, I, J, dtype)
+    X, Wg, Ws, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Ind"))
+    got = hk.expert_mlp_forward(X, Wg, Ws, Ind, "relu", force_block=True)
+    assert got.dtype == dtype and tuple(got.shape) == (B, T, I)
+    assert_close(got, _mlp_oracle(case, T, "relu", dtype), dtype, "inference block")
+    assert torch.equal(got, hk.expert_mlp_forward(X, Wg, Ws, Ind, "relu", force_block=True))     # fixed order of additions
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("act", ["none", "relu", "gelu", "gelu_tanh", "silu"])
+def test_inference_block_activations_and_rejected_picks(act):
+    B, T, E, K, I, J = 8, 96, 16, 24, 128, 64
+    dtype = torch.bfloat16
+    case = make_case(37, B, T, E, K, I, J, dtype, ind_dtype=torch.int16)
+    case["Ind"][0, 0, 0] = T; case["Ind"][1, 2, 3] = -1; case["Ind"][7, 15, 23] = 30000
+    X, Wg, Ws, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Ind"))
+    got = hk.expert_mlp_forward(X, Wg, Ws, Ind, act, force_block=True)
+    assert_close(got, _mlp_oracle(case, T, act, dtype), dtype, f"inference block, {act}")
+    # the same through the two forward launchers with torch's activation in between
+    y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    y = {"none": lambda v: v, "relu": torch.relu, "gelu": torch.nn.functional.gelu, "silu": torch.nn.functional.silu,
+         "gelu_tanh": lambda v: torch.nn.functional.gelu(v, approximate="tanh")}[act](y)
+    two = np64(hk.expert_scatter_forward_call(y, Ws, Ind, T, torch.float32))
+    # the separate launches round Y to bf16 before AND after the activation, the block once; and the block feeds the
+    # reduction elements of the second product to the matrix instruction in another order (fp32 sums differ in the last bit)
+    g64 = np64(got)
+    if act in ("none", "relu"):
+        assert_close(got, two, dtype, f"inference block vs separate launches, {act}")
+    else:
+        assert np.abs(g64 - two).max() <= 4 * 2.0 ** -8 * np.abs(two).max()
+        assert np.sqrt(((g64 - two) ** 2).mean()) <= 8e-3 * np.sqrt((two ** 2).mean())
+
+
+@pytest.mark.gpu
+def test_inference_block_composes_what_the_kernel_does_not_take():
+    # fp32, a 16-bit shape with 2048 picks per batch element, J = 128: same result through the separate launchers
+    for shape, dtype in (((2, 40, 6, 9, 64, 32), torch.float32), ((2, 64, 32, 64, 128, 64), torch.bfloat16),
+                         ((5, 40, 12, 33, 128, 128), torch.float16)):
+        B, T, E, K, I, J = shape
+        case = make_case(41, B, T, E, K, I, J, dtype)
+        X, Wg, Ws, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Ind"))
+        got = hk.expert_mlp_forward(X, Wg, Ws, Ind, "silu")
+        assert_close(got, _mlp_oracle(case, T, "silu", dtype, stored_y=True), dtype, "composed inference block")
+    with pytest.raises(ValueError):
+        hk.expert_mlp_forward(X, Wg, Ws, Ind, "softmax")
