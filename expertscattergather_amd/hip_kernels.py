@@ -329,6 +329,14 @@ def _register_ops(ns: str) -> None:
     lib.define("expert_scatter_forward_call_fn(Tensor Y, Tensor W, Tensor Ind, int T, ScalarType out_dtype) -> Tensor")
     lib.define("expert_scatter_backward_call_fn(Tensor Y, Tensor W, Tensor Ind, Tensor grad_X, "
                "ScalarType out_dtype) -> (Tensor, Tensor)")
+    if ns == OP_NAMESPACE:      # the inference block has no counterpart among the reference's ops
+        lib.define("expert_mlp_forward_fn(Tensor X, Tensor W_gather, Tensor W_scatter, Tensor Ind, str activation, "
+                   "bool force_block=False) -> Tensor")
+        lib.impl("expert_mlp_forward_fn", _mlp_forward_impl, "CompositeExplicitAutograd")
+
+        @torch.library.register_fake(f"{ns}::expert_mlp_forward_fn", lib=lib)
+        def _(X, W_gather, W_scatter, Ind, activation, force_block=False):
+            return X.new_empty(tuple(X.shape))
     lib.impl("expert_gather_forward_call_fn", _gather_forward_impl, "CompositeExplicitAutograd")
     lib.impl("expert_gather_backward_call_fn", _gather_backward_impl, "CompositeExplicitAutograd")
     lib.impl("expert_scatter_forward_call_fn", _scatter_forward_impl, "CompositeExplicitAutograd")
@@ -555,6 +563,18 @@ def _mlp_block_pays(B: int, E: int, I: int, J: int, act: int) -> bool:
 
 def expert_mlp_forward(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor,
                        activation="relu", force_block: bool = False) -> torch.Tensor:
+    """See `_mlp_forward_impl`.  In eager mode on GPU tensors this runs the launcher directly; while torch.compile
+    is tracing (and for fake / meta tensors) it goes through the op ``egs_amd::expert_mlp_forward_fn``, whose fake
+    implementation describes the output."""
+    if type(X) in (torch.Tensor, torch.nn.Parameter) and X.is_cuda and not torch.compiler.is_compiling():
+        return _mlp_forward_impl(X, W_gather, W_scatter, Ind, activation, force_block)
+    create_kernels()
+    return getattr(torch.ops, OP_NAMESPACE).expert_mlp_forward_fn(X, W_gather, W_scatter, Ind,
+                                                                  "none" if activation is None else activation, force_block)
+
+
+def _mlp_forward_impl(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor,
+                      activation="relu", force_block: bool = False) -> torch.Tensor:
     """Inference block ``scatter(act(gather(X, W_gather, Ind)), W_scatter, Ind, T)`` - the call pattern of the
     reference's layers (test_speed.ipynb:73-75 on egs/triton_kernels.py:49-143, :156-247) - without autograd.
 

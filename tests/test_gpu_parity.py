@@ -693,3 +693,20 @@ def test_inference_block_composes_what_the_kernel_does_not_take():
         assert_close(got, _mlp_oracle(case, T, "silu", dtype, stored_y=True), dtype, "composed inference block")
     with pytest.raises(ValueError):
         hk.expert_mlp_forward(X, Wg, Ws, Ind, "softmax")
+
+
+def test_inference_block_is_a_traceable_op():
+    hk.create_kernels()
+    B, T, E, K, I, J = 8, 48, 8, 16, 64, 32
+    dtype = torch.bfloat16
+    case = make_case(43, B, T, E, K, I, J, dtype)
+    X, Wg, Ws, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Ind"))
+    torch.library.opcheck(torch.ops.egs_amd.expert_mlp_forward_fn.default, (X, Wg, Ws, Ind, "relu"),
+                          test_utils=("test_schema", "test_faketensor"))
+    eager = hk.expert_mlp_forward(X, Wg, Ws, Ind, "relu")
+
+    @torch.compile(backend="aot_eager", fullgraph=True)
+    def f(x, wg, ws, ind):
+        return hk.expert_mlp_forward(x, wg, ws, ind, "relu") * 2.0
+
+    assert torch.equal(f(X, Wg, Ws, Ind), eager * 2.0)

@@ -195,3 +195,13 @@ def test_scratch_is_allocated_per_call():
     assert keep.numel() == 1000 and ptr == keep.data_ptr() and n == 1000
     assert not hasattr(hk, "_workspaces")
     hk.release_workspaces()                                           # harmless no-op
+
+
+def test_inference_block_traces_on_meta_tensors():
+    X = torch.empty(2, 5, 64, device="meta", dtype=torch.bfloat16); Wg = torch.empty(4, 64, 32, device="meta", dtype=torch.bfloat16)
+    Ws = torch.empty(4, 32, 64, device="meta", dtype=torch.bfloat16); Ind = torch.empty(2, 4, 3, dtype=torch.int16, device="meta")
+    out = hk.expert_mlp_forward(X, Wg, Ws, Ind, "gelu")
+    assert out.device.type == "meta" and tuple(out.shape) == (2, 5, 64) and out.dtype == torch.bfloat16
+    # the heuristic that chooses between the one kernel and the separate launches
+    assert hk._mlp_block_pays(64, 32, 128, 64, 1) and not hk._mlp_block_pays(64, 32, 128, 64, 2)
+    assert hk._mlp_block_pays(64, 16, 128, 64, 2) and not hk._mlp_block_pays(128, 32, 128, 64, 1)
