@@ -100,7 +100,7 @@ const char *egs_status_string(int status);
 /* text of the last HIP error seen by the calling thread ("" if none) */
 const char *egs_last_hip_error(void);
 
-/* bytes of scratch the op needs for these sizes (0 is a valid answer: small experts in 16-bit types run on
+/* bytes of scratch the op needs for these sizes (0 is a valid answer: small experts run on
  * kernels that keep every intermediate on the CU).  `mode` is an egs_scatter_mode and only matters for ops
  * that scatter.  The answer holds for dense operands that start on a 16-byte boundary (what hipMalloc and
  * torch return); every entry point derives the requirement again from the operands it is given, and an
