@@ -293,6 +293,34 @@ def test_strided_source_rows():
     assert torch.equal(Y, Y2)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bfloat16", "float32"])
+def test_strided_source_rows_on_the_small_expert_kernels(dtype):
+    # rows of X and of the scatter's incoming gradient taken out of wider tensors (token stride 2I + 8 elements, 16-byte
+    # aligned): register-resident gather, one-pass weight gradient in both backward calls, inference block
+    B, T, E, K, I, J = 8, 64, 32, 16, 128, 64
+    case = make_case(19, B, T, E, K, I, J, dtype)
+    def widen(t):
+        big = torch.randn(B, T, 2 * I + 8).to(dtype)
+        big[:, :, 8:8 + I] = t
+        v = dev(big)[:, :, 8:8 + I]
+        assert not v.is_contiguous()
+        return v
+    Xs, dOs = widen(case["X"]), widen(case["dOut"])
+    Wg, Ws, Y, Ind = (dev(case[k]) for k in ("Wg", "Ws", "Y", "Ind"))
+    Xn, Wgn, Wsn, Yn, dOn = (np64(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut"))
+    Indn = case["Ind"].numpy()
+    assert_close(hk.expert_gather_forward_call(Xs, Wg, Ind, torch.float32), O.gather_forward(Xn, Wgn, Indn), dtype, "strided X")
+    dX, dWg = hk.expert_gather_backward_call(Xs, Wg, Ind, Y, torch.float32)
+    rX, rWg = O.gather_backward(Xn, Wgn, Indn, Yn)
+    assert_close(dX, rX, dtype, "dX, strided X"); assert_close(dWg, rWg, dtype, "dWg, strided X")
+    dY, dWs = hk.expert_scatter_backward_call(Y, Ws, Ind, dOs, torch.float32)
+    rY, rWs = O.scatter_backward(Yn, Wsn, Indn, dOn)
+    assert_close(dY, rY, dtype, "dY, strided gradient"); assert_close(dWs, rWs, dtype, "dWs, strided gradient")
+    if dtype is torch.bfloat16:
+        got = hk.expert_mlp_forward(Xs, Wg, Ws, Ind, "relu", force_block=True)
+        assert_close(got, _mlp_oracle(case, T, "relu", dtype), dtype, "inference block, strided X")
+
+
 def test_empty_inputs():
     Wg = torch.zeros(3, 8, 4, device=DEV); Ws = torch.zeros(3, 4, 8, device=DEV)
     X = torch.zeros(2, 5, 8, device=DEV)
