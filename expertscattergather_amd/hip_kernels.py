@@ -552,13 +552,15 @@ _TORCH_ACT = {
 }
 
 
-def _mlp_block_pays(B: int, E: int, I: int, J: int, act: int) -> bool:
+def _mlp_block_pays(B: int, E: int, K: int, I: int, J: int, act: int) -> bool:
     """Measured on MI355X (bf16): the one kernel wins while its workgroups fit one round of the device (256) and the
-    activation is cheap or the experts few; B64 T256 E32 K32 I128 J64: relu 22.8 against 27.3 us, gelu 33.1 against
-    28.9 us; E16: 14.6 / 23.3 us and 21.0 / 23.0 us; B128: 43.3 / 41.6 us."""
+    activation is cheap or the (expert, 32-pick) units few - its four slice workgroups per batch element each repeat
+    the activation, and exponentials run at a quarter of the vector rate.  B64 T256 E32 K32 I128 J64, block / separate
+    launches: relu 22.9 / 27.4 us, silu 26.4 / 27.9, gelu 30.4 / 28.4; E16: 14.5 / 24.8, 17.1 / 24.5, 19.3 / 25.0;
+    B128 relu: 43.3 / 41.6 us."""
     blocks = 8 * ((B + 7) // 8) * (I // 32)
     cheap = act in (_abi.ACT_NONE, _abi.ACT_RELU)
-    return blocks <= 256 and (cheap or E * I * J <= 16 * 128 * 64)
+    return blocks <= 256 and (cheap or E * ((K + 31) // 32) <= 16)
 
 
 def expert_mlp_forward(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor,
@@ -598,7 +600,7 @@ def _mlp_forward_impl(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.
     T = X.shape[1]
     d = _abi.Dims(B, T, E, K, I, J)
     lib = _abi.lib()
-    if ct is not torch.float32 and (force_block or _mlp_block_pays(B, E, I, J, act)) \
+    if ct is not torch.float32 and (force_block or _mlp_block_pays(B, E, K, I, J, act)) \
             and lib.egs_expert_mlp_supported(d, dtype_to_type_id(ct)):
         res_dtype = X.dtype
         Xs, ld_b, ld_t = _rows_source(X, ct)

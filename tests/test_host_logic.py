@@ -203,5 +203,5 @@ def test_inference_block_traces_on_meta_tensors():
     out = hk.expert_mlp_forward(X, Wg, Ws, Ind, "gelu")
     assert out.device.type == "meta" and tuple(out.shape) == (2, 5, 64) and out.dtype == torch.bfloat16
     # the heuristic that chooses between the one kernel and the separate launches
-    assert hk._mlp_block_pays(64, 32, 128, 64, 1) and not hk._mlp_block_pays(64, 32, 128, 64, 2)
-    assert hk._mlp_block_pays(64, 16, 128, 64, 2) and not hk._mlp_block_pays(128, 32, 128, 64, 1)
+    assert hk._mlp_block_pays(64, 32, 32, 128, 64, 1) and not hk._mlp_block_pays(64, 32, 32, 128, 64, 2)
+    assert hk._mlp_block_pays(64, 16, 32, 128, 64, 2) and not hk._mlp_block_pays(128, 32, 32, 128, 64, 1)
