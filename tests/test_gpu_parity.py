@@ -738,3 +738,34 @@ def test_inference_block_is_a_traceable_op():
         return hk.expert_mlp_forward(x, wg, ws, ind, "relu") * 2.0
 
     assert torch.equal(f(X, Wg, Ws, Ind), eager * 2.0)
+
+
+def test_concurrent_callers_on_their_own_streams():
+    # the library keeps no per-call state: two host threads, each on a stream of its own, run different shapes
+    # (different kernels, different LDS grants) at the same time and both get the oracle's answer
+    import threading
+    jobs = [((4, 64, 8, 16, 128, 64), torch.bfloat16), ((2, 256, 48, 32, 128, 64), torch.float16)]
+    cases = [make_case(51 + n, *shape, dtype) for n, (shape, dtype) in enumerate(jobs)]
+    results, errors = [None, None], []
+
+    def worker(n):
+        try:
+            shape, dtype = jobs[n]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    results[n] = run_all(cases[n], shape[1])
+            stream.synchronize()
+        except Exception as exc:            # surfaced in the main thread below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(n,)) for n in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for n, (shape, dtype) in enumerate(jobs):
+        ref = oracle_all(cases[n], shape[1])
+        for name in ("Y", "out", "dX", "dWg", "dY", "dWs"):
+            assert_close(results[n][name], ref[name], dtype, f"thread {n} {name}")
