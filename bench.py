@@ -72,9 +72,11 @@ def parse_args():
     ap.add_argument("--no-cold", action="store_true", help="skip the timing of each launch with the caches flushed in between")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="only launch a 64 MiB device copy (3x) and one entry point of the path (5x), for rocprofv3 --pmc runs")
-    ap.add_argument("--probe-kernel", default="gather", choices=["gather", "scatter", "dw", "scatter_bwd", "gather_bwd"],
+    ap.add_argument("--probe-kernel", default="gather", choices=["gather", "scatter", "dw", "scatter_bwd", "gather_bwd", "mlp", "mlp_separate"],
                     help="which entry point --pmc-probe launches: gather forward, scatter forward, the stand-alone weight "
-                         "gradient, or one of the two backward calls (each shares its launch with a weight gradient)")
+                         "gradient, one of the two backward calls (each shares its launch with a weight gradient), the "
+                         "inference block gather -> relu -> scatter as one kernel (mlp; 16-bit small-expert shapes) or the "
+                         "same as three launches (mlp_separate)")
     return ap.parse_args()
 
 
@@ -125,6 +127,11 @@ def main():
                 hk.expert_scatter_backward_call(Yp, Ws, Ind, dOut, torch.float32)
             elif args.probe_kernel == "gather_bwd":
                 hk.expert_gather_backward_call(X, Wg, Ind, Yp, torch.float32)
+            elif args.probe_kernel == "mlp":
+                hk.expert_mlp_forward(X, Wg, Ws, Ind, "relu", force_block=True)
+            elif args.probe_kernel == "mlp_separate":
+                hk.expert_scatter_forward_call(torch.relu(hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)), Ws, Ind, T,
+                                               torch.float32)
             else:
                 rc = _abi.lib().egs_dw(X.data_ptr(), Yp.data_ptr(), Ind.data_ptr(), dWp.data_ptr(), wsp.data_ptr(), wsb, dp,
                                        T * I, I, dtp, dtp, _abi.IND_I64, _abi.W_EIJ, torch.cuda.current_stream().cuda_stream)
