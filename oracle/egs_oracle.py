@@ -18,6 +18,9 @@ reference defines in plain torch:
 * scatter backward -- the transposed identities the reference realises by swapping W
                       strides at ``egs/triton_kernels.py:504`` (dY) and ``:521`` (dW).
 
+* inference block   -- the two forwards chained through an elementwise activation, the way the
+                      reference's notebook calls its layers (``test_speed.ipynb:73-75``).
+
 How each function is pinned (the reference ships no golden vectors for this path, its
 tests are unseeded random GPU comparisons, ``test_all.py:97-101``):
 
@@ -166,6 +169,45 @@ def scatter_backward(Y, W, Ind, dOut, acc=np.float64):
 
 
 # ----------------------------------------------------------------------------- brute force
+# ---------------------------------------------------------------------------------------------------------
+# Inference block: the reference's layers chained the way its notebook calls them, out = scatter(act(gather(x, Ind)), Ind, T)
+# (test_speed.ipynb:73-75 with gather = egs/baselines.py:69-76 and scatter = egs/baselines.py:174-184).
+def activation(y, name):
+    """Elementwise activations by their textbook closed forms (float64): relu, gelu (erf form, the default of
+    torch.nn.functional.gelu), gelu_tanh (its tanh approximation), silu, none.  Pinned in tests/test_oracle.py against
+    torch.nn.functional on the CPU and against special values."""
+    y = np.asarray(y, dtype=np.float64)
+    if name in (None, "none", "identity"):
+        return y
+    if name == "relu":
+        return np.maximum(y, 0.0)
+    if name == "gelu":
+        from math import erf
+        return 0.5 * y * (1.0 + np.vectorize(erf, otypes=[np.float64])(y / np.sqrt(2.0)))
+    if name == "gelu_tanh":
+        return 0.5 * y * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (y + 0.044715 * y ** 3)))
+    if name == "silu":
+        return y / (1.0 + np.exp(-y))
+    raise ValueError(f"unknown activation {name!r}")
+
+
+def mlp_forward(X, Wg, Ws, Ind, T, act="relu", round_y=None, round_before_act=False):
+    """out = scatter_forward(act(gather_forward(X, Wg, Ind)), Ws, Ind, T), picks outside [0, T) contributing nothing.
+
+    `round_y`: function that rounds the activated rows to the element type a stored Y would have (e.g. round_to_bf16), or
+    None.  `round_before_act`: also round before the activation, as separate launches that store Y do."""
+    Ind = _as_index(np.asarray(Ind))
+    bad = (Ind < 0) | (Ind >= T)
+    safe = np.where(bad, 0, Ind)
+    Y = gather_forward(X, Wg, safe)
+    if round_y is not None and round_before_act:
+        Y = round_y(Y.astype(np.float32)).astype(np.float64)
+    Y = activation(Y, act) * (~bad)[..., None]
+    if round_y is not None:
+        Y = round_y(Y.astype(np.float32)).astype(np.float64)
+    return scatter_forward(Y, Ws, safe, T)
+
+
 def brute_gather_forward(X, W, Ind):
     """Index-by-index restatement of the summation formula (tiny shapes only)."""
     B, T, I = X.shape

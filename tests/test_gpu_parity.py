@@ -631,32 +631,12 @@ def test_modules_trace_through_torch_compile():
 
 # ---------------------------------------------------------------------------------------------------------
 # inference block: scatter(act(gather(x, Ind)), Ind, T) in one kernel (reference call pattern test_speed.ipynb:73-75)
-def _np_act(y, name):
-    from scipy.special import erf
-    if name == "relu":
-        return np.maximum(y, 0.0)
-    if name == "gelu":
-        return 0.5 * y * (1.0 + erf(y / np.sqrt(2.0)))
-    if name == "gelu_tanh":
-        return 0.5 * y * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (y + 0.044715 * y ** 3)))
-    if name == "silu":
-        return y / (1.0 + np.exp(-y))
-    return y
-
-
 def _mlp_oracle(case, T, act, dtype, stored_y=False):
-    """The oracle's gather, the activation in float64, one rounding to the element type where a stored Y would be
-    rounded, the oracle's scatter.  `stored_y`: Y is also rounded before the activation (separate launches)."""
+    """oracle/egs_oracle.py mlp_forward with the rows rounded to the element type where a stored Y would be rounded
+    (`stored_y`: also before the activation, as the separate launches do)."""
+    rnd = lambda v: torch.from_numpy(v).to(dtype).to(torch.float32).numpy()
     X, Wg, Ws = (np64(case[k]) for k in ("X", "Wg", "Ws"))
-    Ind = case["Ind"].numpy()
-    bad = (Ind < 0) | (Ind >= T)
-    safe = np.where(bad, 0, Ind)
-    Y = O.gather_forward(X, Wg, safe)
-    if stored_y:
-        Y = np64(torch.from_numpy(Y).to(dtype))
-    Y = _np_act(Y, act) * (~bad)[..., None]
-    Y = np64(torch.from_numpy(Y).to(dtype))
-    return O.scatter_forward(Y, Ws, safe, T)
+    return O.mlp_forward(X, Wg, Ws, case["Ind"].numpy(), T, act, round_y=rnd, round_before_act=stored_y)
 
 
 MLP_SHAPES = [

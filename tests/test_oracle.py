@@ -205,3 +205,54 @@ def test_fp8_encoder_and_row_quantiser_match_torch():
     q2, xs2 = O.quantize_rows_e4m3(Xn)
     bad = np.zeros(xs.shape, dtype=bool); bad[0, 0] = bad[3, 2] = bad[6, 4] = True
     assert np.isnan(xs2[bad]).all() and np.array_equal(xs2[~bad], xs[~bad]) and np.array_equal(q2[~bad], q[~bad])
+
+
+# ---------------------------------------------------------------------------------------------------------
+# inference block: activation closed forms and the chained forward
+def test_activations_against_torch_and_special_values():
+    y = np.linspace(-9.0, 9.0, 721)
+    t = torch.from_numpy(y)
+    F = torch.nn.functional
+    for name, fn in (("relu", torch.relu), ("gelu", F.gelu), ("silu", F.silu),
+                     ("gelu_tanh", lambda v: F.gelu(v, approximate="tanh")), ("none", lambda v: v)):
+        np.testing.assert_allclose(O.activation(y, name), fn(t).numpy(), rtol=1e-12, atol=1e-14, err_msg=name)
+    # what the mathematics fixes: zero at zero, identity far to the right, zero (relu) or vanishing far to the left,
+    # gelu(x) - gelu(-x) = x and silu(x) - silu(-x) = x (the even parts cancel)
+    for name in ("relu", "gelu", "gelu_tanh", "silu"):
+        assert O.activation(np.array([0.0]), name)[0] == 0.0
+        assert abs(O.activation(np.array([30.0]), name)[0] - 30.0) < 1e-9
+        assert abs(O.activation(np.array([-30.0]), name)[0]) < 1e-9
+    for name in ("gelu", "gelu_tanh", "silu"):
+        np.testing.assert_allclose(O.activation(y, name) - O.activation(-y, name), y, rtol=0, atol=1e-12)
+    assert abs(O.activation(np.array([1.0]), "gelu")[0] - 0.8413447460685429) < 1e-15      # Phi(1)
+    assert abs(O.activation(np.array([1.0]), "silu")[0] - 0.7310585786300049) < 1e-15      # 1 / (1 + 1/e)
+    with pytest.raises(ValueError):
+        O.activation(y, "softmax")
+
+
+def test_inference_block_is_the_chain_of_the_two_forwards():
+    rng = np.random.default_rng(5)
+    B, T, E, K, I, J = 2, 7, 3, 4, 5, 6
+    X = rng.standard_normal((B, T, I)); Wg = rng.standard_normal((E, I, J)); Ws = rng.standard_normal((E, J, I))
+    Ind = rng.integers(0, T, (B, E, K))
+    Ind[0, 1, 2] = T + 3; Ind[1, 0, 0] = -1                              # rejected picks contribute nothing
+    bad = (Ind < 0) | (Ind >= T)
+    for act in ("none", "relu", "gelu", "silu"):
+        # index-by-index: rows of Y for the valid picks only, activated, multiplied and added where they belong
+        out = np.zeros((B, T, I))
+        for b in range(B):
+            for e in range(E):
+                for k in range(K):
+                    if bad[b, e, k]:
+                        continue
+                    y = O.activation(X[b, Ind[b, e, k]] @ Wg[e], act)
+                    out[b, Ind[b, e, k]] += y @ Ws[e]
+        np.testing.assert_allclose(O.mlp_forward(X, Wg, Ws, Ind, T, act), out, rtol=1e-12, atol=1e-12)
+    # without an activation the block is linear in X; with rounding hooks the rows pass through them
+    a = O.mlp_forward(X, Wg, Ws, Ind, T, "none"); b2 = O.mlp_forward(2.5 * X, Wg, Ws, Ind, T, "none")
+    np.testing.assert_allclose(b2, 2.5 * a, rtol=1e-12, atol=1e-12)
+    calls = []
+    def spy(v):
+        calls.append(v.shape); return v
+    O.mlp_forward(X, Wg, Ws, Ind, T, "relu", round_y=spy, round_before_act=True)
+    assert calls == [(B, E, K, J), (B, E, K, J)]
