@@ -61,6 +61,18 @@ def main():
     Ind = g.integers(0, 6, size=(2, 3, 4)).astype(np.int64)
     blob.update({"fp8/X": X, "fp8/Wq_bits": bits, "fp8/scale": scale, "fp8/Ind": Ind,
                  "fp8/gather_Y": O.gather_forward_fp8w(X, bits, scale, Ind)})
+    # inference block (gather -> activation -> scatter), bf16 inputs, rows rounded to bf16 after the activation; one
+    # rejected pick; a shape the one-kernel form takes (8 batch elements, I = J = 32)
+    g = np.random.default_rng(91)
+    B, T, E, K, I, J = 8, 12, 4, 6, 32, 32
+    X = O.round_to_bf16(g.standard_normal((B, T, I)).astype(np.float32))
+    Wg = O.round_to_bf16((g.standard_normal((E, I, J)) / np.sqrt(I)).astype(np.float32))
+    Ws = O.round_to_bf16((g.standard_normal((E, J, I)) / np.sqrt(J)).astype(np.float32))
+    Ind = g.integers(0, T, size=(B, E, K)).astype(np.int32)
+    Ind[3, 2, 1] = T + 1
+    blob.update({"mlp/X": X, "mlp/Wg": Wg, "mlp/Ws": Ws, "mlp/Ind": Ind})
+    for act in ("relu", "silu", "gelu"):
+        blob[f"mlp/out_{act}"] = O.mlp_forward(X, Wg, Ws, Ind, T, act, round_y=O.round_to_bf16)
     path = os.path.join(HERE, "egs_golden.npz")
     np.savez_compressed(path, **blob)
     print(path, os.path.getsize(path), "bytes,", len(blob), "arrays")

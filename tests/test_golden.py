@@ -13,7 +13,7 @@ from tests._util import assert_close
 
 PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "egs_golden.npz")
 GOLD = np.load(PATH)
-CASES = sorted({k.split("/")[0] for k in GOLD.files} - {"fp8"})
+CASES = sorted({k.split("/")[0] for k in GOLD.files} - {"fp8", "mlp"})
 DTYPE = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 
@@ -42,6 +42,26 @@ def test_fp8_fixture():
     np.testing.assert_array_equal(O.gather_forward_fp8w(c["X"], c["Wq_bits"], c["scale"], c["Ind"]), c["gather_Y"])
     W = torch.from_numpy(c["Wq_bits"]).view(torch.float8_e4m3fn).double().numpy() * c["scale"].astype(np.float64)[:, None, :]
     np.testing.assert_allclose(O.gather_forward(c["X"], W, c["Ind"]), c["gather_Y"], rtol=1e-12, atol=1e-15)
+
+
+def test_inference_block_fixture():
+    c = case("mlp")
+    T = c["X"].shape[1]
+    for act in ("relu", "silu", "gelu"):
+        np.testing.assert_array_equal(O.mlp_forward(c["X"], c["Wg"], c["Ws"], c["Ind"], T, act, round_y=O.round_to_bf16),
+                                      c[f"out_{act}"])
+
+
+@pytest.mark.gpu
+def test_hip_inference_block_matches_the_fixture():
+    from expertscattergather_amd import hip_kernels as hk
+    c = case("mlp")
+    dev = "cuda"
+    t = lambda a: torch.from_numpy(a).to(dev, torch.bfloat16)
+    Ind = torch.from_numpy(c["Ind"]).to(dev)
+    for act in ("relu", "silu", "gelu"):
+        got = hk.expert_mlp_forward(t(c["X"]), t(c["Wg"]), t(c["Ws"]), Ind, act, force_block=True)
+        assert_close(got, c[f"out_{act}"], torch.bfloat16, f"inference block {act}")
 
 
 @pytest.mark.gpu
