@@ -158,3 +158,20 @@ def test_inference_block_entry_point_validates_without_a_gpu(lib):
                                       _abi.ACT_RELU, None) == _abi.EGS_ERR_UNSUPPORTED
     assert lib.egs_expert_mlp_forward(p, p, p, p, p + 2, ok, 256 * 128, 128, _abi.BF16, _abi.IND_I64, _abi.ACT_RELU,
                                       None) == _abi.EGS_ERR_UNSUPPORTED                                # output off the 16-byte grid
+
+
+def test_planning_functions_survive_arbitrary_sizes(lib):
+    # the size queries run the same selection code as the entry points: whatever the sizes, they answer (no
+    # division by zero, no overflow into nonsense), in multiples of 256 bytes, and agree with themselves
+    import random
+    rnd = random.Random(3)
+    pick = lambda: rnd.choice([0, 1, 2, 3, 7, 8, 16, 31, 32, 33, 64, 100, 128, 256, 300, 512, 1024, 4096, 65536, 2 ** 31 - 1])
+    for _ in range(3000):
+        d = _abi.Dims(pick(), pick(), pick(), pick(), pick(), pick())
+        for dt in (_abi.F32, _abi.F16, _abi.BF16):
+            sizes = [lib.egs_workspace_bytes(op, mode, d, dt) for op in range(5) for mode in (0, 1)]
+            assert all(s % 256 == 0 for s in sizes), (tuple(getattr(d, f) for f in "BTEKIJ"), sizes)
+            assert sizes == [lib.egs_workspace_bytes(op, mode, d, dt) for op in range(5) for mode in (0, 1)]
+            assert lib.egs_expert_mlp_supported(d, dt) in (0, 1)
+        assert lib.egs_gather_gemm_fp8act_workspace_bytes(d) % 256 == 0
+    assert lib.egs_workspace_bytes(1, 0, None, _abi.BF16) == 0 and lib.egs_expert_mlp_supported(None, _abi.BF16) == 0
