@@ -184,3 +184,18 @@ def test_c5_fp8_activations_forward():
         rel_rms = np.sqrt(((np64(Y[b, e]) - ref) ** 2).mean() / (ref ** 2).mean())
         assert rel_rms <= 5e-2, rel_rms
     assert torch.equal(Y, hk.expert_gather_fp8_forward(Xg, Wqg, sg, Ig))
+
+
+def test_c2_inference_block_full_size():
+    # gather -> relu -> scatter of the default shape in one kernel against the oracle's chained forward (rows rounded to
+    # bf16 where a stored Y would be), repeated bit for bit, tokens nobody picked exactly zero
+    cfg, inp, g = gpu_inputs("C2")
+    B, T, E, K, I, J = cfg.dims
+    got = hk.expert_mlp_forward(g["X"], g["Wg"], g["Ws"], g["Ind"], "relu", force_block=True)
+    ref = O.mlp_forward(np64(inp["X"]), np64(inp["Wg"]), np64(inp["Ws"]), inp["Ind"].numpy(), T, "relu",
+                        round_y=O.round_to_bf16)
+    assert_close(got, ref, torch.bfloat16, "C2 inference block")
+    assert torch.equal(got, hk.expert_mlp_forward(g["X"], g["Wg"], g["Ws"], g["Ind"], "relu", force_block=True))
+    picked = torch.zeros(B, T, dtype=torch.bool)
+    picked.scatter_(1, inp["Ind"].reshape(B, -1).long(), True)
+    assert float(got.cpu()[~picked].abs().max() if (~picked).any() else 0.0) == 0.0
