@@ -33,8 +33,8 @@ PROFILES = os.path.join(ROOT, "profiles")
 # kernel (as rocprofv3 names it) behind each launch of the path, per workload; where a call runs several kernels
 # the one that takes most of its time is named and the others are listed in the profile summaries
 LAUNCH_KERNELS = {
-    "C2": {"expert_gather_forward": "rows_small_kernel", "expert_scatter_forward": "scatter_fused_kernel",
-           "expert_scatter_backward": "rows_dw_tile_kernel", "expert_gather_backward": "scatter_fused_dwtile_kernel"},
+    "C2": {"expert_gather_forward": "rows_small_kernel", "expert_scatter_forward": "scatter_fused_table_kernel",
+           "expert_scatter_backward": "rows_dw_tile_kernel", "expert_gather_backward": "scatter_fused_dwtile_table_kernel"},
     "C1": {"expert_gather_forward": "rows_small_f32_kernel", "expert_scatter_forward": "scatter_fused_kernel"},
     "C3": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel",
            "expert_scatter_backward": "rows_gemm_dl_kernel + dw_dl_kernel", "expert_gather_backward": "rows_gemm_dl_kernel + segment_sum_kernel + dw_dl_kernel"},
@@ -120,6 +120,7 @@ def main():
             if args.config == "C5":
                 hk.expert_gather_fp8w_forward(X, Wq_p, scale_p, Ind)
             elif args.probe_kernel == "gather":
+                hk.invalidate_routing_table(Ind)        # every dispatch builds the routing table, as the first of a step does
                 hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
             elif args.probe_kernel == "scatter":
                 hk.expert_scatter_forward_call(Yp, Ws, Ind, T, torch.float32)
@@ -150,6 +151,9 @@ def main():
         Wq, Wscale = Wq_c.to(dev), scale_c.to(dev)
 
     def step():
+        # a training step routes anew: the table that the gather forward leaves with Ind for the scatter forward and the
+        # gather's backward is rebuilt in every step, never carried over from the step before
+        hk.invalidate_routing_table(Ind)
         if fp8_act:
             Y = hk.expert_gather_fp8_forward(X, Wq, Wscale, Ind)
         elif fp8:
@@ -219,6 +223,10 @@ def main():
     f8ws_bytes = lib.egs_gather_gemm_fp8act_workspace_bytes(d) if fp8_act else 0
     f8ws = torch.empty(max(f8ws_bytes, 256), dtype=torch.uint8, device=dev)
     I64 = _abi.IND_I64
+    # the launches as a step issues them: where the sizes have a routing table, the gather forward builds it and the
+    # scatter forward and the gather's backward read it
+    tab_bytes = 0 if fp8 else lib.egs_routing_table_bytes(d, dt)
+    tab = torch.empty(max(tab_bytes, 256), dtype=torch.uint8, device=dev)
 
     def k_gather():
         if fp8_act:     # row quantiser + fp8 x fp8 product: both launches are part of the call
@@ -227,9 +235,15 @@ def main():
         if fp8:
             return lib.egs_gather_gemm(X.data_ptr(), Wq.data_ptr(), Ind.data_ptr(), Y.data_ptr(), Wscale.data_ptr(), d, T * I, I, dt,
                                        _abi.FP8_E4M3, I64, _abi.W_EIJ, stream)
+        if tab_bytes:
+            return lib.egs_expert_gather_forward_table(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), tab.data_ptr(),
+                                                       tab_bytes, d, T * I, I, dt, I64, stream)
         return lib.egs_expert_gather_forward(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d, T * I, I, dt, I64, stream)
 
     def k_scatter():
+        if tab_bytes:
+            return lib.egs_expert_scatter_forward_table(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), tab.data_ptr(), tab_bytes,
+                                                        out.data_ptr(), ws.data_ptr(), ws_bytes, d, dt, I64, mode, stream)
         return lib.egs_expert_scatter_forward(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), out.data_ptr(), ws.data_ptr(), ws_bytes, d,
                                               dt, I64, mode, stream)
 
@@ -238,6 +252,10 @@ def main():
                                                dWs_b.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, I64, stream)
 
     def k_gather_bwd():
+        if tab_bytes:
+            return lib.egs_expert_gather_backward_table(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), tab.data_ptr(), tab_bytes,
+                                                        dYb.data_ptr(), dXb.data_ptr(), dWg_b.data_ptr(), ws.data_ptr(), ws_bytes,
+                                                        d, T * I, I, dt, I64, mode, stream)
         return lib.egs_expert_gather_backward(X.data_ptr(), Wg.data_ptr(), Ind.data_ptr(), dYb.data_ptr(), dXb.data_ptr(),
                                               dWg_b.data_ptr(), ws.data_ptr(), ws_bytes, d, T * I, I, dt, I64, mode, stream)
 
@@ -283,6 +301,7 @@ def main():
     if not fwd_only:
         launches["expert_scatter_backward"] = (k_scatter_bwd, gemm_bytes + dw_bytes, 2 * kflops)
         launches["expert_gather_backward"] = (k_gather_bwd, gemm_bytes + dw_bytes, 2 * kflops)
+    assert k_gather() == 0      # the table is in place before the launches that read it are timed
     warm = {name: time_kernel(fn, reps) for name, (fn, _, _) in launches.items()}
     cold = None if flush is None else {name: time_kernel_cold(fn, 10) for name, (fn, _, _) in launches.items()}
     dw_alone_s = None if fwd_only else time_kernel(k_dw, reps)
@@ -371,6 +390,7 @@ def main():
         "step_tflops": round(chain_flops / step_s * 1e-12, 2),
         "eager_us_per_step": round(eager_s * 1e6, 2),
         "graph_us_per_step": None if graph_s is None else round(graph_s * 1e6, 2),
+        "routing_table_bytes": int(tab_bytes),
         "launch_us": {k: round(v * 1e6, 2) for k, v in warm.items()},
         "launch_us_cold": None if cold is None else {k: round(v * 1e6, 2) for k, v in cold.items()},
         "dw_alone_us": None if dw_alone_s is None else round(dw_alone_s * 1e6, 2),

@@ -221,8 +221,13 @@ struct DwTileJob {
     bool done;          // set once it has been enqueued
 };
 
+// A routing table in caller-owned memory (egs_routing_table_bytes): seg [B][T+1], perm [B][E*K], the picks of each batch
+// element in a stable order by token.  Built once per Ind by a gather forward, read by the one-kernel scatters that follow.
+struct RoutingTable { int32_t *seg, *perm; };
+
 bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
-                       int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, SmallRowsJob &j)
+                       int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, SmallRowsJob &j,
+                       const RoutingTable *build = nullptr)
 {
     const int R = d->I, N = d->J;
     if (g_force_generic || w_dtype != act_dtype || !small_shape_ok(act_dtype, R, N)) return false;
@@ -248,7 +253,12 @@ bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, c
     }
     j.R = R; j.act_dtype = act_dtype; j.gather = true; j.out_f32 = false; j.lds = 0;
     j.nmajor = (w_layout == EGS_W_EIJ);                 // [E,I,J] = [E,R,N]
-    j.blocks = p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e;
+    if (build != nullptr) {             // the routing table of a later scatter rides along: B more workgroups, first in line
+        p.csr_blocks = d->B;
+        p.seg_off = build->seg; p.perm = build->perm;
+        j.lds = csr_count_lds(d->T, 4);
+    }
+    j.blocks = (p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e) + p.csr_blocks;
     return true;
 }
 
@@ -607,6 +617,24 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
                                            "hipFuncSetAttribute(scatter_fused_multi_kernel)");
         if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_multi_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
+    } else if (p.tab_seg != nullptr && dwt != nullptr && !dwt->wide && TT::ES == 2) {
+      if constexpr (TT::ES == 2) {
+        static LdsGrant told_dwt_tab;
+        const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
+        const size_t need = lds > tile_lds ? lds : tile_lds;
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_dwtile_table_kernel<TT, W_NMAJOR, KS>, told_dwt_tab, need,
+                                           "hipFuncSetAttribute(scatter_fused_dwtile_table_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
+        hipLaunchKernelGGL((scatter_fused_dwtile_table_kernel<TT, W_NMAJOR, KS>), dim3(blocks + dwt->blocks), dim3(kFusedThreads), need,
+                           s, p, dwt->q, blocks);
+        dwt->done = true;
+      }
+    } else if (p.tab_seg != nullptr && dw == nullptr && (dwt == nullptr || dwt->wide || TT::ES != 2)) {
+        static LdsGrant told_tab;
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_table_kernel<TT, W_NMAJOR, KS>, told_tab, lds,
+                                           "hipFuncSetAttribute(scatter_fused_table_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
+        hipLaunchKernelGGL((scatter_fused_table_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     } else if (dwt != nullptr && !dwt->wide) {
       if constexpr (TT::ES == 2) {
         const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
@@ -688,7 +716,7 @@ bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const eg
 // GEMM-scatter of small experts in one kernel; the caller has checked scatter_fused_takes().  Both scatter modes
 // take it: it is bitwise reproducible and needs no workspace.
 int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
-                  int w_layout, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s)
+                  int w_layout, SmallDwJob *dw, DwTileJob *dwt, hipStream_t s, const RoutingTable *use = nullptr)
 {
     const int R = d->J, N = d->I;
     const int64_t NP = (int64_t)d->E * d->K;
@@ -704,6 +732,7 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.ind_dtype = ind_dtype;
     p.slices = slices;
     p.experts_per_pass = fp.experts_per_pass;
+    if (use != nullptr && fp.experts_per_pass == d->E && NP <= 1024 && d->T + 1 <= 2048) { p.tab_seg = use->seg; p.tab_perm = use->perm; }
     p.perm_at = (int32_t)((int64_t)fp.experts_per_pass * d->K * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
@@ -745,16 +774,52 @@ size_t scatter_bytes_planned(const egs_dims *d, int mode, int act_dtype)
     return plan_scatter(d, mode, act_dtype, scatter_fused_takes(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype)).bytes;
 }
 
+// Layout of a caller-owned routing table, for the sizes whose one-kernel scatter can read one (16-bit types, one pass,
+// T + 1 <= 2048 table offsets per batch element); `ok` false: a table would not be used.
+struct TableLayout { bool ok; size_t perm_at, bytes; };
+TableLayout routing_table_layout(const egs_dims *d, int act_dtype)
+{
+    TableLayout l = {false, 0, 0};
+    if (!(act_dtype == EGS_F16 || act_dtype == EGS_BF16)) return l;
+    const FusedPlan fp = scatter_fused_plan(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype);
+    if (!fp.ok || fp.experts_per_pass != d->E || d->T + 1 > 2048) return l;
+    l.ok = true;
+    l.perm_at = align_up((size_t)d->B * (d->T + 1) * 4, 256);
+    l.bytes = l.perm_at + align_up((size_t)d->B * d->E * d->K * 4, 256);
+    return l;
+}
+
+// checks a table argument of an entry point; fills `t` when the table is to be used
+int check_table_arg(void *table, size_t table_bytes, const egs_dims *d, int act_dtype, RoutingTable &t, bool &have)
+{
+    have = false;
+    if (table == nullptr) return EGS_OK;
+    const TableLayout l = routing_table_layout(d, act_dtype);
+    if (!l.ok) return EGS_ERR_UNSUPPORTED;
+    if (!aligned_to(table, 256)) return EGS_ERR_ALIGNMENT;
+    if (table_bytes < l.bytes) return EGS_ERR_WORKSPACE;
+    t.seg = (int32_t *)table;
+    t.perm = (int32_t *)((char *)table + l.perm_at);
+    have = true;
+    return EGS_OK;
+}
+
 // ------------------------------------------------------------------------------ implementations
 int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, const float *w_scale,
                      const egs_dims *d, int64_t ldx_b, int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype,
-                     int w_layout, hipStream_t s)
+                     int w_layout, hipStream_t s, const RoutingTable *build = nullptr)
 {
     const int ES = elem_size(act_dtype), WES = elem_size(w_dtype);
     if (w_scale == nullptr) {
         SmallRowsJob j;
-        if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j))
+        if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j, build))
             return launch_rows_small_job(j, nullptr, nullptr, s);
+    }
+    if (build != nullptr) {             // no launch for the table to ride in: a launch of its own
+        const int rc = launch_routing_table(Ind, ind_dtype, d, build->seg, build->perm, nullptr, nullptr, nullptr, s);
+        if (rc != EGS_OK) return rc;
+    }
+    if (w_scale == nullptr) {
         if (act_dtype == EGS_F32 && w_dtype == EGS_F32) {
             bool used = false;
             const int rc = gather_small_f32(X, W, Ind, Y, d, ldx_b, ldx_t, ind_dtype, w_layout, s, used);
@@ -785,7 +850,7 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
 // launch and whose second pass may share the reduction launch
 int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, void *workspace,
                       const egs_dims *d, int act_dtype, int ind_dtype, int w_layout, int mode, SmallDwJob *dw,
-                      DwTileJob *dwt, hipStream_t s)
+                      DwTileJob *dwt, hipStream_t s, const RoutingTable *use = nullptr)
 {
     const int ES = elem_size(act_dtype);
     const size_t out_elems = (size_t)d->B * d->T * d->I;
@@ -820,7 +885,7 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
         return rows_gemm_scatter(p, act_dtype, w_trans, EPI_ATOMIC_F32, s);
     }
 
-    if (fused) return scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s);    // small experts: one kernel
+    if (fused) return scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s, use);   // small experts: one kernel
 
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
     // gather-and-sum per token that writes every output row exactly once
@@ -1097,17 +1162,21 @@ int egs_expert_gather_forward(const void *X, const void *W, const void *Ind, voi
     return egs_gather_gemm(X, W, Ind, Y, nullptr, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, stream);
 }
 
-int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, const void *grad_Y,
-                               void *grad_X, void *grad_W,
-                               void *workspace, size_t workspace_bytes, const egs_dims *d,
-                               int64_t ldx_b, int64_t ldx_t,
-                               int dtype, int ind_dtype, int mode, void *stream)
+static int gather_backward_impl(const void *X, const void *W, const void *Ind, const void *grad_Y,
+                                void *grad_X, void *grad_W,
+                                void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                int64_t ldx_b, int64_t ldx_t,
+                                int dtype, int ind_dtype, int mode, void *stream, void *table, size_t table_bytes)
 {
     int rc = check_dims(d);
     if (rc != EGS_OK) return rc;
     if (!act_dtype_ok(dtype)) return EGS_ERR_BAD_DTYPE;
     if (!mode_ok(mode)) return EGS_ERR_BAD_MODE;
     if (grad_X == nullptr && (size_t)d->B * d->T * d->I > 0) return EGS_ERR_NULL_POINTER;
+    RoutingTable tab;
+    bool have_tab = false;
+    rc = check_table_arg(table, table_bytes, d, dtype, tab, have_tab);
+    if (rc != EGS_OK) return rc;
     const size_t ws_scatter = plan_scatter(d, mode, dtype, scatter_fused_takes(grad_Y, W, grad_X, d, dtype)).bytes;
     const size_t ws_dw = (size_t)d->B * d->K > 0 && (size_t)d->E * d->I * d->J > 0 && grad_W != nullptr
         ? dw_choose(X, grad_Y, grad_W, d, ldx_b, ldx_t, dtype, plan_dw(d, dtype)).bytes : 0;
@@ -1135,7 +1204,7 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     const bool dw_small = !dw_tile && w_elems > 0 && make_dw_small(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype,
                                                                    ind_dtype, EGS_W_EIJ, dpl, dwj);
     rc = gemm_scatter_impl(grad_Y, W, Ind, grad_X, workspace, d, dtype, ind_dtype, EGS_W_EIJ, mode, dw_small ? &dwj : nullptr,
-                           dw_tile ? &dwt : nullptr, s);
+                           dw_tile ? &dwt : nullptr, s, have_tab ? &tab : nullptr);
     if (rc != EGS_OK) return rc;
     if (w_elems == 0) return EGS_OK;
     if (dw_tile) return dwt.done ? EGS_OK : launch_dw_tile_alone(dwt, s);
@@ -1146,11 +1215,67 @@ int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, co
     return dw_general(X, grad_Y, Ind, grad_W, ws2, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, dpl, s);
 }
 
+int egs_expert_gather_backward(const void *X, const void *W, const void *Ind, const void *grad_Y,
+                               void *grad_X, void *grad_W,
+                               void *workspace, size_t workspace_bytes, const egs_dims *d,
+                               int64_t ldx_b, int64_t ldx_t,
+                               int dtype, int ind_dtype, int mode, void *stream)
+{
+    return gather_backward_impl(X, W, Ind, grad_Y, grad_X, grad_W, workspace, workspace_bytes, d, ldx_b, ldx_t, dtype, ind_dtype,
+                                mode, stream, nullptr, 0);
+}
+
+int egs_expert_gather_backward_table(const void *X, const void *W, const void *Ind, const void *table, size_t table_bytes,
+                                     const void *grad_Y, void *grad_X, void *grad_W,
+                                     void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                     int64_t ldx_b, int64_t ldx_t,
+                                     int dtype, int ind_dtype, int mode, void *stream)
+{
+    return gather_backward_impl(X, W, Ind, grad_Y, grad_X, grad_W, workspace, workspace_bytes, d, ldx_b, ldx_t, dtype, ind_dtype,
+                                mode, stream, const_cast<void *>(table), table_bytes);
+}
+
 int egs_expert_scatter_forward(const void *Y, const void *W, const void *Ind, void *Out,
                                void *workspace, size_t workspace_bytes, const egs_dims *d,
                                int dtype, int ind_dtype, int mode, void *stream)
 {
     return egs_gemm_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, dtype, ind_dtype, EGS_W_EJI, mode, stream);
+}
+
+int egs_expert_scatter_forward_table(const void *Y, const void *W, const void *Ind, const void *table, size_t table_bytes,
+                                     void *Out, void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                     int dtype, int ind_dtype, int mode, void *stream)
+{
+    int rc = validate_scatter(Y, W, Ind, Out, workspace, workspace_bytes, d, dtype, ind_dtype, EGS_W_EJI, mode);
+    if (rc != EGS_OK) return rc;
+    RoutingTable tab;
+    bool have_tab = false;
+    rc = check_table_arg(const_cast<void *>(table), table_bytes, d, dtype, tab, have_tab);
+    if (rc != EGS_OK) return rc;
+    return gemm_scatter_impl(Y, W, Ind, Out, workspace, d, dtype, ind_dtype, EGS_W_EJI, mode, nullptr, nullptr,
+                             (hipStream_t)stream, have_tab ? &tab : nullptr);
+}
+
+size_t egs_routing_table_bytes(const egs_dims *d, int dtype)
+{
+    if (check_dims(d) != EGS_OK) return 0;
+    const TableLayout l = routing_table_layout(d, dtype);
+    return l.ok ? l.bytes : 0;
+}
+
+int egs_expert_gather_forward_table(const void *X, const void *W, const void *Ind, void *Y, void *table, size_t table_bytes,
+                                    const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                                    int dtype, int ind_dtype, void *stream)
+{
+    int rc = validate_gather(X, W, Ind, Y, nullptr, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ);
+    if (rc != EGS_OK) return rc;
+    RoutingTable tab;
+    bool have_tab = false;
+    rc = check_table_arg(table, table_bytes, d, dtype, tab, have_tab);
+    if (rc != EGS_OK) return rc;
+    if ((size_t)d->B * d->E * d->K * d->J == 0) return EGS_OK;
+    return gather_gemm_impl(X, W, Ind, Y, nullptr, d, ldx_b, ldx_t, dtype, dtype, ind_dtype, EGS_W_EIJ, (hipStream_t)stream,
+                            have_tab ? &tab : nullptr);
 }
 
 int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, const void *grad_Out,

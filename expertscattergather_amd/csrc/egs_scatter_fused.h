@@ -46,6 +46,9 @@ struct ScatterFusedParams {
     int32_t slices;         // N / kFusedCols
     int32_t perm_at, cnt_at;    // byte offsets of the table and of the sort's counters in dynamic LDS (rows start at 0)
     int32_t experts_per_pass;   // MULTI: experts whose product rows are in LDS at a time (E otherwise)
+    // TABLE: routing table built beforehand (seg [B][T+1], perm [B][E*K]); the workgroup copies its batch element's part
+    // into LDS instead of sorting the picks itself
+    const int32_t *tab_seg, *tab_perm;
 };
 
 constexpr int kFusedMaxPasses = 4;
@@ -59,7 +62,7 @@ __host__ __device__ inline size_t scatter_fused_lds(int T, int NP, int rows)
 }
 __host__ __device__ inline size_t scatter_fused_lds(int T, int NP) { return scatter_fused_lds(T, NP, NP); }
 
-template <class TT, bool W_NMAJOR, int KS, bool MULTI = false>
+template <class TT, bool W_NMAJOR, int KS, bool MULTI = false, bool TABLE = false>
 __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, const int block, char *smem)
 {
     // KS = reduction length in MFMA steps of four 16-byte chunks: 32 elements of a 16-bit type, 16 of fp32
@@ -185,10 +188,31 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     // ---------------- (0) routing table of batch element b in LDS; the first units' operands go in flight
     // right behind the sort's token loads and travel while it runs
     const int EP = MULTI ? p.experts_per_pass : E;
+    if constexpr (TABLE) {
+        // the table comes from memory: its loads go first, the operands behind them; it is parked in LDS in the places
+        // the sort would have left it while the operands travel (NP <= 1024, T < 2048: checked by the host)
+        constexpr int PV = 1024 / kFusedThreads, SV = 2048 / kFusedThreads;
+        const int32_t *gseg = p.tab_seg + (size_t)b * (T + 1), *gperm = p.tab_perm + (size_t)b * NP;
+        int32_t pv[PV], sv[SV];
+#pragma unroll
+        for (int x = 0; x < PV; ++x) pv[x] = gperm[min(tid + x * kFusedThreads, NP - 1)];
+#pragma unroll
+        for (int x = 0; x < SV; ++x) sv[x] = gseg[min(tid + x * kFusedThreads, T)];
+#pragma unroll
+        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, E);
+        int32_t *seg_w = cnt + NWV * T;
+#pragma unroll
+        for (int x = 0; x < PV; ++x)
+            if (tid + x * kFusedThreads < NP) perm[tid + x * kFusedThreads] = pv[x];
+#pragma unroll
+        for (int x = 0; x < SV; ++x)
+            if (tid + x * kFusedThreads <= T) seg_w[tid + x * kFusedThreads] = sv[x];
+    } else {
     csr_count_body(cnt, b, 0, tid, kFusedThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr, [&]() {
 #pragma unroll
         for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
     });
+    }
 
     const int cc = tid & 7;
     auto store_row = [&](int t, const f32x4 &sum) {
@@ -316,6 +340,25 @@ __global__ __launch_bounds__(kFusedThreads) void scatter_fused_dw_kernel(Scatter
         scatter_fused_body<TT, W_NMAJOR, KS>(p, (int)blockIdx.x, smem_fused_dw);
     } else {
         dw_small_body<TT, kFusedThreads / 64>(q, (int)blockIdx.x - fused_blocks, reinterpret_cast<float *>(smem_fused_dw));
+    }
+}
+
+// with the routing table read from memory instead of sorted in the kernel
+template <class TT, bool W_NMAJOR, int KS>
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_table_kernel(ScatterFusedParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_fused_table[];
+    scatter_fused_body<TT, W_NMAJOR, KS, false, true>(p, (int)blockIdx.x, smem_fused_table);
+}
+
+template <class TT, bool W_NMAJOR, int KS>
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_dwtile_table_kernel(ScatterFusedParams p, DwTileParams q, int fused_blocks)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_fused_dwtile_table[];
+    if ((int)blockIdx.x < fused_blocks) {
+        scatter_fused_body<TT, W_NMAJOR, KS, false, true>(p, (int)blockIdx.x, smem_fused_dwtile_table);
+    } else {
+        if constexpr (TT::ES == 2) dw_tile_body<TT, kFusedThreads / 64>(q, (int)blockIdx.x - fused_blocks, smem_fused_dwtile_table);
     }
 }
 

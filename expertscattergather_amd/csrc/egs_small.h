@@ -54,15 +54,13 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     constexpr int R = 32 * KS;
     constexpr int OES = OUT_F32 ? 4 : 2;        // output element size
     static_assert(!(GATHER && OUT_F32), "gather results are stored in the element type");
-    if constexpr (!GATHER) {
-        if (block < p.csr_blocks) {
-            csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
-                           p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
-            return;
-        }
+    if (block < p.csr_blocks) {             // uniform per workgroup; 0 unless a routing table rides along
+        csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
+                       p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
+        return;
     }
     int e, tile;
-    const int bid = block - (GATHER ? 0 : p.csr_blocks);
+    const int bid = block - p.csr_blocks;
     if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
                          : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: scalar address work

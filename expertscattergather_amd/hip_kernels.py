@@ -27,6 +27,7 @@ __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
     "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
     "register_reference_namespace", "release_workspaces", "expert_mlp_forward",
+    "set_routing_table_cache", "invalidate_routing_table",
 ]
 
 OP_NAMESPACE = "egs_amd"
@@ -219,6 +220,64 @@ def _compute_dtype(out_dtype: torch.dtype, *tensors: torch.Tensor) -> torch.dtyp
     return out_dtype
 
 
+# ------------------------------------------------------------------------------ routing table kept with Ind
+# The one-kernel scatter of small experts sorts the picks of a batch element by token before it adds product rows in a
+# fixed order.  That order is a function of Ind alone, so the gather forward - the first call of a layer that sees Ind -
+# builds it in its own launch (a few extra workgroups) and leaves it with the Ind tensor OBJECT; the scatter forward and
+# the gather's backward that are handed the same object, unchanged, read it instead of sorting again.  The entry is
+# tied to the object's data pointer, shape, dtype, version counter, T and stream, so it dies with the tensor and
+# is ignored after any in-place write that autograd can see.  A write that bypasses the version counter (a custom
+# kernel through data_ptr, `Ind.data`'s own counter) is not seen - the same blind spot autograd's saved-tensor check has;
+# call invalidate_routing_table(Ind) after such a write, or set_routing_table_cache(False).  Nothing is attached or read
+# while the stream is being captured into a graph (the table's memory would belong to the graph's pool).
+_TABLE_ATTR = "_egs_routing_table"
+_table_cache = os.environ.get("EGS_ROUTING_TABLE_CACHE", "1") != "0"
+_table_sizes: dict = {}
+
+
+def set_routing_table_cache(enabled: bool) -> None:
+    """Switch the reuse of routing tables between calls that share an Ind tensor on or off (default on,
+    EGS_ROUTING_TABLE_CACHE=0 turns it off); results are bit-identical either way."""
+    global _table_cache
+    _table_cache = bool(enabled)
+
+
+def invalidate_routing_table(Ind: torch.Tensor) -> None:
+    """Forget the routing table kept with `Ind` (after writing into it through a channel its version counter does not see)."""
+    Ind.__dict__.pop(_TABLE_ATTR, None)
+
+
+def _table_key(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
+    return (Ind.data_ptr(), Ind._version, Ind.dtype, dims, dt, stream)
+
+
+def _table_nbytes(dims: tuple, dt: int) -> int:
+    key = (dims, dt)
+    n = _table_sizes.get(key)
+    if n is None:
+        n = _table_sizes[key] = int(_abi.lib().egs_routing_table_bytes(_abi.Dims(*dims), dt))
+    return n
+
+
+def _table_wanted(Ind: torch.Tensor, dims: tuple, dt: int) -> int:
+    """Bytes of the table these sizes can use, or 0 when none is to be built or read now."""
+    if not _table_cache or dt == _abi.F32 or type(Ind) is not torch.Tensor:
+        return 0
+    n = _table_nbytes(dims, dt)
+    if n == 0 or torch.cuda.is_current_stream_capturing():
+        return 0
+    return n
+
+
+def _table_lookup(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
+    if _table_wanted(Ind, dims, dt) == 0:
+        return None
+    ent = Ind.__dict__.get(_TABLE_ATTR)
+    if ent is None or ent[0] != _table_key(Ind, dims, dt, stream):
+        return None
+    return ent[1]
+
+
 # ------------------------------------------------------------------------------ the four launchers
 def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     ct = _compute_dtype(out_dtype, X, W)
@@ -228,10 +287,23 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     X, ld_b, ld_t = _rows_source(X, ct)
     W = _dense16(W, ct); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
-    d = _abi.Dims(B, X.shape[1], E, K, I, J)
+    T = X.shape[1]
+    d = _abi.Dims(B, T, E, K, I, J)
+    dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
-                                                  ld_b, ld_t, dtype_to_type_id(ct), _ind_type_id(Ind), _stream_ptr(dev))
+        stream = _stream_ptr(dev)
+        dims = (B, T, E, K, I, J)
+        nb = _table_wanted(Ind, dims, dt)
+        if nb and _table_lookup(Ind, dims, dt, stream) is None:
+            # first sight of these indices: the routing table of the scatters to come is built in this launch
+            table = torch.empty(nb, dtype=torch.uint8, device=dev)
+            rc = _abi.lib().egs_expert_gather_forward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
+                                                            table.data_ptr(), nb, d, ld_b, ld_t, dt, _ind_type_id(Ind), stream)
+            if rc == 0:
+                Ind.__dict__[_TABLE_ATTR] = (_table_key(Ind, dims, dt, stream), table)
+        else:
+            rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
+                                                      ld_b, ld_t, dt, _ind_type_id(Ind), stream)
     if rc:
         _abi.check(rc, "expert_gather_forward_call")
     return Y if res_dtype is ct else Y.to(res_dtype)
@@ -252,9 +324,17 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, (B, T, E, K, I, J), dt))
-        rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
-                                                   grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
-                                                   dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+        stream = _stream_ptr(dev)
+        table = _table_lookup(Ind, (B, T, E, K, I, J), dt, stream)
+        if table is not None:
+            rc = _abi.lib().egs_expert_gather_backward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
+                                                             table.numel(), grad_output.data_ptr(), grad_X.data_ptr(),
+                                                             grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t, dt,
+                                                             _ind_type_id(Ind), mode, stream)
+        else:
+            rc = _abi.lib().egs_expert_gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_output.data_ptr(),
+                                                       grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
+                                                       dt, _ind_type_id(Ind), mode, stream)
     del keep
     if rc:
         _abi.check(rc, "expert_gather_backward_call")
@@ -276,8 +356,15 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, (B, T, E, K, I, J), dt))
-        rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
-                                                   ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, _stream_ptr(dev))
+        stream = _stream_ptr(dev)
+        table = _table_lookup(Ind, (B, T, E, K, I, J), dt, stream)
+        if table is not None:
+            rc = _abi.lib().egs_expert_scatter_forward_table(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
+                                                             table.numel(), out.data_ptr(), ws, ws_bytes, d, dt,
+                                                             _ind_type_id(Ind), mode, stream)
+        else:
+            rc = _abi.lib().egs_expert_scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), out.data_ptr(),
+                                                       ws, ws_bytes, d, dt, _ind_type_id(Ind), mode, stream)
     del keep
     if rc:
         _abi.check(rc, "expert_scatter_forward_call")

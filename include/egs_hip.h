@@ -176,6 +176,41 @@ int egs_gather_gemm_fp8act(const void *X, const void *Wq, const float *w_scale, 
                            int64_t ldx_b, int64_t ldx_t, int ind_dtype, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Routing table in caller-owned memory (new; the reference has nothing of the kind: its scatter kernel adds with
+ * atomics, egs/triton_kernels.py:247).  The one-kernel scatter of small experts sorts the picks of a batch element by
+ * token before it can add product rows in a fixed order; Ind decides that order alone, so it can be computed once per
+ * Ind and reused by every scatter over the same Ind: the scatter forward, and the scatter inside the gather's backward.
+ *   - egs_routing_table_bytes(): size of the table for these sizes, 0 if no kernel would read one (then pass no table).
+ *   - egs_expert_gather_forward_table(): egs_expert_gather_forward, and fills `table` from Ind in the same launch
+ *     (a launch of its own when the operands do not select the small-expert gather).
+ *   - egs_expert_scatter_forward_table(), egs_expert_gather_backward_table(): the plain entry points with a table that
+ *     was filled from the SAME Ind contents and the same sizes; results are bit-identical to the plain entry points.
+ *     The table is only read.  A table built from other indices gives wrong sums without any error: the caller owns
+ *     that invariant.
+ * `table` NULL makes each of these the plain entry point.  A table argument for sizes that have no use for one returns
+ * EGS_ERR_UNSUPPORTED; `table` must be 256-byte aligned (EGS_ERR_ALIGNMENT) and at least egs_routing_table_bytes() long
+ * (EGS_ERR_WORKSPACE).
+ * ------------------------------------------------------------------------------------- */
+size_t egs_routing_table_bytes(const egs_dims *d, int dtype);
+
+int egs_expert_gather_forward_table(const void *X, const void *W, const void *Ind, void *Y,
+                                    void *table, size_t table_bytes,
+                                    const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
+                                    int dtype, int ind_dtype, void *stream);
+
+int egs_expert_scatter_forward_table(const void *Y, const void *W, const void *Ind,
+                                     const void *table, size_t table_bytes, void *Out,
+                                     void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                     int dtype, int ind_dtype, int mode, void *stream);
+
+int egs_expert_gather_backward_table(const void *X, const void *W, const void *Ind,
+                                     const void *table, size_t table_bytes,
+                                     const void *grad_Y, void *grad_X, void *grad_W,
+                                     void *workspace, size_t workspace_bytes, const egs_dims *d,
+                                     int64_t ldx_b, int64_t ldx_t,
+                                     int dtype, int ind_dtype, int mode, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Inference block (new; no single kernel of the reference corresponds to it): the reference's call pattern
  *   out = scatter(act(gather(x, Ind)), Ind, T)          (test_speed.ipynb:73-75)
  * in ONE kernel for small experts; the rows Y[B,E,K,J] between the two products stay in registers:

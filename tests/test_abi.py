@@ -160,6 +160,31 @@ def test_inference_block_entry_point_validates_without_a_gpu(lib):
                                       None) == _abi.EGS_ERR_UNSUPPORTED                                # output off the 16-byte grid
 
 
+def test_routing_table_entry_points_validate_without_a_gpu(lib):
+    tb = lib.egs_routing_table_bytes
+    d = _abi.Dims(64, 256, 32, 32, 128, 64)
+    seg, perm = -(-64 * 257 * 4 // 256) * 256, 64 * 32 * 32 * 4
+    assert tb(d, _abi.BF16) == tb(d, _abi.F16) == seg + perm                # [B][T + 1] offsets, then [B][E * K] picks
+    assert tb(d, _abi.F32) == 0                                              # fp32 scatters read no table
+    assert tb(_abi.Dims(64, 256, 48, 32, 128, 64), _abi.BF16) == 0           # scatter in passes sorts per pass
+    assert tb(_abi.Dims(16, 256, 8, 640, 128, 64), _abi.BF16) == 0           # general path builds its own in the workspace
+    assert tb(None, _abi.BF16) == 0 and tb(d, 9) == 0
+    p, t, nb = 0x1000, 0x4000, seg + perm
+    gf, sf, gb = lib.egs_expert_gather_forward_table, lib.egs_expert_scatter_forward_table, lib.egs_expert_gather_backward_table
+    ld = (256 * 128, 128)
+    assert gf(p, p, p, p, t, nb - 1, d, *ld, _abi.BF16, _abi.IND_I64, None) == -6            # table too small
+    assert gf(p, p, p, p, t + 16, nb, d, *ld, _abi.BF16, _abi.IND_I64, None) == -7           # not 256-byte aligned
+    assert gf(p, p, p, p, t, nb, d, *ld, _abi.F32, _abi.IND_I64, None) == _abi.EGS_ERR_UNSUPPORTED
+    assert gf(None, p, p, p, t, nb, d, *ld, _abi.BF16, _abi.IND_I64, None) == -1
+    assert sf(p, p, p, t, nb - 1, p, None, 0, d, _abi.BF16, _abi.IND_I64, 0, None) == -6
+    assert sf(p, p, p, t, nb, p, None, 0, d, _abi.F32, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
+    assert sf(p, p, p, t, nb, p, None, 0, d, _abi.BF16, _abi.IND_I64, 7, None) == -5          # unknown mode
+    assert gb(p, p, p, t, nb - 1, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -6
+    assert gb(p, p, p, t + 16, nb, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -7
+    big = _abi.Dims(64, 256, 48, 32, 128, 64)
+    assert gb(p, p, p, t, nb, p, p, p, None, 0, big, *ld, _abi.BF16, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
+
+
 def test_planning_functions_survive_arbitrary_sizes(lib):
     # the size queries run the same selection code as the entry points: whatever the sizes, they answer (no
     # division by zero, no overflow into nonsense), in multiples of 256 bytes, and agree with themselves
@@ -173,5 +198,6 @@ def test_planning_functions_survive_arbitrary_sizes(lib):
             assert all(s % 256 == 0 for s in sizes), (tuple(getattr(d, f) for f in "BTEKIJ"), sizes)
             assert sizes == [lib.egs_workspace_bytes(op, mode, d, dt) for op in range(5) for mode in (0, 1)]
             assert lib.egs_expert_mlp_supported(d, dt) in (0, 1)
+            assert lib.egs_routing_table_bytes(d, dt) % 256 == 0
         assert lib.egs_gather_gemm_fp8act_workspace_bytes(d) % 256 == 0
     assert lib.egs_workspace_bytes(1, 0, None, _abi.BF16) == 0 and lib.egs_expert_mlp_supported(None, _abi.BF16) == 0

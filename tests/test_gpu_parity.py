@@ -95,10 +95,12 @@ SMALL_SHAPES = [
 def force_generic(request):
     from expertscattergather_amd import _abi
     _abi.lib().egs_testing_force_generic(1 if request.param else 0)
-    hk._ws_sizes.clear()                    # remembered workspace sizes belong to the other kernel family
+    hk._ws_sizes.clear()                    # remembered workspace and table sizes belong to the other kernel family
+    hk._table_sizes.clear()
     yield request.param
     _abi.lib().egs_testing_force_generic(0)
     hk._ws_sizes.clear()
+    hk._table_sizes.clear()
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d).split(".")[-1])

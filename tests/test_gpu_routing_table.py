@@ -1,0 +1,196 @@
+"""The routing table that the gather forward leaves with an Ind tensor for the scatter forward and the gather's backward:
+results are the same bit for bit with and without it, the table is the stable sort of the picks by token, and it is never
+used for indices other than the ones it was built from."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import egs_oracle as O
+from tests._util import assert_close, make_case, np64
+
+pytestmark = pytest.mark.gpu
+
+from expertscattergather_amd import _abi
+from expertscattergather_amd import hip_kernels as hk
+
+hk.create_kernels()
+DEV = "cuda"
+ATTR = hk._TABLE_ATTR
+
+# 16-bit shapes the one-kernel scatter takes in a single pass (the only consumers of a table)
+TABLE_SHAPES = [
+    (2, 256, 32, 32, 128, 64),      # two batch elements of the default shape
+    (5, 50, 9, 11, 64, 32),         # ragged K, T, E
+    (2, 33, 5, 64, 128, 64),
+    (4, 300, 40, 25, 96, 32),       # 1000 picks per batch element
+    (8, 700, 8, 20, 32, 64),        # long T
+    (9, 20, 3, 7, 32, 32),
+]
+
+
+@pytest.fixture(autouse=True)
+def cache_on():
+    hk.set_routing_table_cache(True)
+    yield
+    hk.set_routing_table_cache(True)
+
+
+def chain(case, T, ind=None):
+    """gather forward -> scatter forward -> gather backward, the three calls that share a table."""
+    X, Wg, Ws, Y = (case[k].to(DEV) for k in ("X", "Wg", "Ws", "Y"))
+    Ind = case["Ind"].to(DEV) if ind is None else ind
+    y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+    out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    dX, dWg = hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)
+    torch.cuda.synchronize()
+    return Ind, (y, out, dX, dWg)
+
+
+@pytest.mark.parametrize("ind_dtype", [torch.int64, torch.int16], ids=["i64", "i16"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("shape", TABLE_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_results_do_not_depend_on_the_table(shape, dtype, ind_dtype):
+    B, T, E, K, I, J = shape
+    case = make_case(31 + sum(shape), *shape, dtype, ind_dtype=ind_dtype)
+    hk.set_routing_table_cache(False)
+    ind0, plain = chain(case, T)
+    assert ATTR not in ind0.__dict__
+    hk.set_routing_table_cache(True)
+    ind1, tabled = chain(case, T)
+    assert ATTR in ind1.__dict__, "these sizes have a table: the gather forward must have left one"
+    for a, b, name in zip(plain, tabled, ("Y", "out", "dX", "dWg")):
+        assert torch.equal(a, b), f"{name} differs with the table {shape} {dtype}"
+    assert_close(tabled[1], O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].to(torch.int64).numpy(), T), dtype, "out")
+
+
+def test_table_is_the_stable_sort_of_the_picks_by_token():
+    B, T, E, K, I, J = 5, 50, 9, 11, 64, 32
+    case = make_case(3, B, T, E, K, I, J, torch.bfloat16)
+    Ind = case["Ind"].clone()
+    Ind[1, 2, 3] = T; Ind[2, 0, 0] = -5         # rejected picks have no place in any token's list
+    X, Wg, IndD = case["X"].to(DEV), case["Wg"].to(DEV), Ind.to(DEV)
+    d = _abi.Dims(B, T, E, K, I, J)
+    nb = _abi.lib().egs_routing_table_bytes(d, _abi.BF16)
+    assert nb > 0
+    table = torch.full((nb,), 0xEE, dtype=torch.uint8, device=DEV)
+    Y = torch.empty(B, E, K, J, dtype=torch.bfloat16, device=DEV)
+    rc = _abi.lib().egs_expert_gather_forward_table(X.data_ptr(), Wg.data_ptr(), IndD.data_ptr(), Y.data_ptr(), table.data_ptr(), nb,
+                                                    d, T * I, I, _abi.BF16, _abi.IND_I64, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    words = table.cpu().numpy().view(np.int32)
+    perm_at = -(-(B * (T + 1) * 4) // 256) * 256 // 4
+    seg = words[:B * (T + 1)].reshape(B, T + 1)
+    perm = words[perm_at:perm_at + B * E * K].reshape(B, E * K)
+    flat = Ind.numpy().reshape(B, E * K)
+    for b in range(B):
+        valid = (flat[b] >= 0) & (flat[b] < T)
+        counts = np.bincount(flat[b][valid], minlength=T)
+        assert (seg[b] == np.concatenate([[0], np.cumsum(counts)])).all()
+        order = np.argsort(np.where(valid, flat[b], T), kind="stable")[:valid.sum()]
+        assert (perm[b, :valid.sum()] == order).all()
+
+
+def test_in_place_writes_to_ind_retire_the_table():
+    shape = (2, 64, 8, 16, 128, 64)
+    B, T, E, K, I, J = shape
+    case = make_case(41, *shape, torch.bfloat16)
+    other = make_case(42, *shape, torch.bfloat16)["Ind"]
+    assert not torch.equal(other, case["Ind"])
+    hk.set_routing_table_cache(False)
+    _, want = chain(dict(case, Ind=other), T)
+    hk.set_routing_table_cache(True)
+    Ind, _ = chain(case, T)
+    assert ATTR in Ind.__dict__
+    Ind.copy_(other.to(DEV))            # same object, same address, new contents: the version counter moves
+    Y, Ws, X, Wg = (case[k].to(DEV) for k in ("Y", "Ws", "X", "Wg"))
+    out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    dX, dWg = hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)
+    assert torch.equal(out, want[1]) and torch.equal(dX, want[2]) and torch.equal(dWg, want[3])
+    # the next gather forward builds the table of the new contents
+    _, again = chain(case, T, ind=Ind)
+    for a, b in zip(again, want):
+        assert torch.equal(a, b)
+    # single elements too
+    Ind[0, 0, 0] = (int(Ind[0, 0, 0]) + 1) % T
+    hk.set_routing_table_cache(False)
+    _, want2 = chain(case, T, ind=Ind.clone())
+    hk.set_routing_table_cache(True)
+    out2 = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    assert torch.equal(out2, want2[1])
+
+
+def test_a_table_serves_only_the_sizes_and_stream_it_was_built_for():
+    shape = (2, 64, 8, 16, 128, 64)
+    B, T, E, K, I, J = shape
+    case = make_case(43, *shape, torch.bfloat16)
+    Ind, _ = chain(case, T)
+    Y, Ws = case["Y"].to(DEV), case["Ws"].to(DEV)
+    # a scatter into more tokens than the gather read from: other sizes, no table
+    T2 = T + 16
+    out = hk.expert_scatter_forward_call(Y, Ws, Ind, T2, torch.float32)
+    assert_close(out, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].numpy(), T2), torch.bfloat16, "other T")
+    # another stream: its launches are not ordered after the launch that builds the table
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert hk._table_lookup(Ind, shape, _abi.BF16, hk._stream_ptr(Ind.device)) is None
+        out_side = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    side.synchronize()
+    hk.set_routing_table_cache(False)
+    want = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+    assert torch.equal(out_side, want)
+    # explicit invalidation
+    hk.set_routing_table_cache(True)
+    assert ATTR in Ind.__dict__
+    hk.invalidate_routing_table(Ind)
+    assert ATTR not in Ind.__dict__
+
+
+def test_no_table_for_fp32_multi_pass_or_under_capture():
+    for shape, dtype in [((2, 64, 8, 16, 128, 64), torch.float32), ((2, 256, 48, 32, 128, 64), torch.bfloat16)]:
+        case = make_case(44, *shape, dtype)
+        Ind, _ = chain(case, shape[1])
+        assert ATTR not in Ind.__dict__
+    shape = (2, 64, 8, 16, 128, 64)
+    case = make_case(45, *shape, torch.bfloat16)
+    X, Wg, Ws, Y, Ind = (case[k].to(DEV) for k in ("X", "Wg", "Ws", "Y", "Ind"))
+    eager_y = hk.expert_gather_forward_call(X, Wg, Ind.clone(), torch.float32)
+    eager_out = hk.expert_scatter_forward_call(Y, Ws, Ind.clone(), shape[1], torch.float32)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        gy = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        gout = hk.expert_scatter_forward_call(Y, Ws, Ind, shape[1], torch.float32)
+    assert ATTR not in Ind.__dict__, "nothing is left with Ind by a captured call"
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gy, eager_y) and torch.equal(gout, eager_out)
+
+
+def test_autograd_chain_uses_and_survives_the_table():
+    import expertscattergather_amd as egs
+    B, T, E, K, I, J = 4, 64, 8, 16, 128, 64
+    torch.manual_seed(0)
+    g = egs.ExpertGather(E, I, J).to(DEV).bfloat16()
+    s = egs.ExpertScatter(E, J, I).to(DEV).bfloat16()
+    x = torch.randn(B, T, I, device=DEV, dtype=torch.bfloat16, requires_grad=True)
+    Ind = torch.randint(0, T, (B, E, K), device=DEV)
+
+    def run():
+        for p in (x, g.W, s.W):
+            p.grad = None
+        out = s(torch.relu(g(x, Ind)), Ind, T)
+        out.float().square().sum().backward()
+        return out.detach().clone(), x.grad.clone(), g.W.grad.clone(), s.W.grad.clone()
+
+    hk.set_routing_table_cache(False)
+    want = run()
+    hk.set_routing_table_cache(True)
+    got = run()
+    assert ATTR in Ind.__dict__
+    again = run()                   # second step with the same Ind object: the table is found, not rebuilt
+    for a, b, c in zip(want, got, again):
+        assert torch.equal(a, b) and torch.equal(a, c)
