@@ -54,6 +54,7 @@ SIGNATURES = {
     "egs_expert_scatter_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _vp]),
     "egs_validate_indices": (_i, [_vp, _i, _i64, ctypes.c_int32, _vp, _vp]),
     "egs_routing_table_bytes": (_sz, [_dp, _i]),
+    "egs_stream_capture_id": (_i, [_vp, ctypes.POINTER(ctypes.c_ulonglong)]),
     "egs_expert_gather_forward_table": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _vp]),
     "egs_expert_scatter_forward_table": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp, _sz, _dp, _i, _i, _i, _vp]),
     "egs_expert_gather_backward_table": (_i, [_vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _dp, _i64, _i64, _i, _i, _i, _vp]),

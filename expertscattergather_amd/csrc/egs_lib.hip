@@ -783,6 +783,12 @@ TableLayout routing_table_layout(const egs_dims *d, int act_dtype)
     if (!(act_dtype == EGS_F16 || act_dtype == EGS_BF16)) return l;
     const FusedPlan fp = scatter_fused_plan(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype);
     if (!fp.ok || fp.experts_per_pass != d->E || d->T + 1 > 2048) return l;
+    // the table pays only when its build rides in the gather forward's launch (as a launch of its own it costs more than
+    // the two scatters save): the register-resident gather must take these sizes too
+    SmallRowsJob gj;
+    if (!make_gather_small(kStandInPtr, kStandInPtr, kStandInPtr, kStandInPtr, d, (int64_t)d->T * d->I, d->I, act_dtype,
+                           act_dtype, EGS_IND_I32, EGS_W_EIJ, gj))
+        return l;
     l.ok = true;
     l.perm_at = align_up((size_t)d->B * (d->T + 1) * 4, 256);
     l.bytes = l.perm_at + align_up((size_t)d->B * d->E * d->K * 4, 256);
@@ -1334,6 +1340,18 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
         if (rc != EGS_OK) return rc;
     }
     return dw_impl(grad_Out, Y, Ind, grad_W, workspace, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, s);
+}
+
+int egs_stream_capture_id(void *stream, unsigned long long *id)
+{
+    if (id == nullptr) return EGS_ERR_NULL_POINTER;
+    *id = 0;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long cid = 0;
+    const hipError_t err = hipStreamGetCaptureInfo((hipStream_t)stream, &status, &cid);
+    if (err != hipSuccess) return hip_fail(err, "hipStreamGetCaptureInfo");
+    if (status == hipStreamCaptureStatusActive) *id = cid;
+    return EGS_OK;
 }
 
 int egs_validate_indices(const void *Ind, int ind_dtype, int64_t n, int32_t T, int32_t *d_bad_count, void *stream)

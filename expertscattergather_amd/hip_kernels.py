@@ -16,6 +16,7 @@ so that ``torch.compile`` can trace through them.
 """
 from __future__ import annotations
 
+import ctypes
 import os
 import threading
 
@@ -146,6 +147,17 @@ def _dense16(t: torch.Tensor, ct: torch.dtype) -> torch.Tensor:
 
 
 _ws_sizes: dict = {}
+_dims_structs: dict = {}
+
+
+def _dims_struct(dims: tuple):
+    """The egs_dims structure of a problem, built once per problem (the library only reads it)."""
+    d = _dims_structs.get(dims)
+    if d is None:
+        if len(_dims_structs) > 4096:
+            _dims_structs.clear()
+        d = _dims_structs[dims] = _abi.Dims(*dims)
+    return d
 
 
 def _workspace_bytes(op: int, mode: int, dims: tuple, dt: int) -> int:
@@ -228,8 +240,10 @@ def _compute_dtype(out_dtype: torch.dtype, *tensors: torch.Tensor) -> torch.dtyp
 # tied to the object's data pointer, shape, dtype, version counter, T and stream, so it dies with the tensor and
 # is ignored after any in-place write that autograd can see.  A write that bypasses the version counter (a custom
 # kernel through data_ptr, `Ind.data`'s own counter) is not seen - the same blind spot autograd's saved-tensor check has;
-# call invalidate_routing_table(Ind) after such a write, or set_routing_table_cache(False).  Nothing is attached or read
-# while the stream is being captured into a graph (the table's memory would belong to the graph's pool).
+# call invalidate_routing_table(Ind) after such a write, or set_routing_table_cache(False).  A table filled by a launch
+# that is being captured into a graph holds nothing until the graph is replayed, and lives in the graph's memory pool: the
+# entry carries the capture's identifier and serves only calls recorded into the same capture (replays rebuild it from
+# whatever Ind then holds, because the launch that fills it is part of the graph).
 _TABLE_ATTR = "_egs_routing_table"
 _table_cache = os.environ.get("EGS_ROUTING_TABLE_CACHE", "1") != "0"
 _table_sizes: dict = {}
@@ -247,8 +261,18 @@ def invalidate_routing_table(Ind: torch.Tensor) -> None:
     Ind.__dict__.pop(_TABLE_ATTR, None)
 
 
-def _table_key(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
-    return (Ind.data_ptr(), Ind._version, Ind.dtype, dims, dt, stream)
+def _capture_id(stream: int) -> int:
+    """0 outside graph capture, the capture's identifier inside one, -1 if it cannot be told (then: no table)."""
+    if not torch.cuda.is_current_stream_capturing():
+        return 0
+    cid = ctypes.c_ulonglong(0)
+    if _abi.lib().egs_stream_capture_id(stream, ctypes.byref(cid)) != 0 or cid.value == 0:
+        return -1
+    return int(cid.value)
+
+
+def _table_key(Ind: torch.Tensor, dims: tuple, dt: int, stream: int, capture: int):
+    return (Ind.data_ptr(), Ind._version, Ind.dtype, dims, dt, stream, capture)
 
 
 def _table_nbytes(dims: tuple, dt: int) -> int:
@@ -259,23 +283,25 @@ def _table_nbytes(dims: tuple, dt: int) -> int:
     return n
 
 
-def _table_wanted(Ind: torch.Tensor, dims: tuple, dt: int) -> int:
-    """Bytes of the table these sizes can use, or 0 when none is to be built or read now."""
+def _table_state(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
+    """(bytes of the table these sizes can use - 0: build and read none now -, capture identifier, the table kept with
+    `Ind` if it is valid for this call else None)."""
     if not _table_cache or dt == _abi.F32 or type(Ind) is not torch.Tensor:
-        return 0
-    n = _table_nbytes(dims, dt)
-    if n == 0 or torch.cuda.is_current_stream_capturing():
-        return 0
-    return n
+        return 0, 0, None
+    nb = _table_nbytes(dims, dt)
+    if nb == 0:
+        return 0, 0, None
+    capture = _capture_id(stream)
+    if capture < 0:
+        return 0, 0, None
+    ent = Ind.__dict__.get(_TABLE_ATTR)
+    if ent is not None and ent[0] == (Ind.data_ptr(), Ind._version, Ind.dtype, dims, dt, stream, capture):
+        return nb, capture, ent[1]
+    return nb, capture, None
 
 
 def _table_lookup(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
-    if _table_wanted(Ind, dims, dt) == 0:
-        return None
-    ent = Ind.__dict__.get(_TABLE_ATTR)
-    if ent is None or ent[0] != _table_key(Ind, dims, dt, stream):
-        return None
-    return ent[1]
+    return _table_state(Ind, dims, dt, stream)[2]
 
 
 # ------------------------------------------------------------------------------ the four launchers
@@ -288,19 +314,19 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     W = _dense16(W, ct); Ind = Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     T = X.shape[1]
-    d = _abi.Dims(B, T, E, K, I, J)
+    dims = (B, T, E, K, I, J)
+    d = _dims_struct(dims)
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         stream = _stream_ptr(dev)
-        dims = (B, T, E, K, I, J)
-        nb = _table_wanted(Ind, dims, dt)
-        if nb and _table_lookup(Ind, dims, dt, stream) is None:
+        nb, capture, table = _table_state(Ind, dims, dt, stream)
+        if nb and table is None:
             # first sight of these indices: the routing table of the scatters to come is built in this launch
             table = torch.empty(nb, dtype=torch.uint8, device=dev)
             rc = _abi.lib().egs_expert_gather_forward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
                                                             table.data_ptr(), nb, d, ld_b, ld_t, dt, _ind_type_id(Ind), stream)
             if rc == 0:
-                Ind.__dict__[_TABLE_ATTR] = (_table_key(Ind, dims, dt, stream), table)
+                Ind.__dict__[_TABLE_ATTR] = (_table_key(Ind, dims, dt, stream, capture), table)
         else:
             rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
                                                       ld_b, ld_t, dt, _ind_type_id(Ind), stream)
@@ -319,13 +345,14 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     T = X.shape[1]
     grad_X = torch.empty((B, T, I), device=dev, dtype=ct)
     grad_W = torch.empty((E, I, J), device=dev, dtype=ct)
-    d = _abi.Dims(B, T, E, K, I, J)
+    dims = (B, T, E, K, I, J)
+    d = _dims_struct(dims)
     mode = _MODES[_scatter_mode]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, (B, T, E, K, I, J), dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, dims, dt))
         stream = _stream_ptr(dev)
-        table = _table_lookup(Ind, (B, T, E, K, I, J), dt, stream)
+        table = _table_state(Ind, dims, dt, stream)[2]
         if table is not None:
             rc = _abi.lib().egs_expert_gather_backward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
                                                              table.numel(), grad_output.data_ptr(), grad_X.data_ptr(),
@@ -351,13 +378,14 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     res_dtype = Y.dtype
     Y = _dense16(Y, ct); W = _dense16(W, ct); Ind = Ind.contiguous()
     out = torch.empty((B, T, I), device=dev, dtype=ct)
-    d = _abi.Dims(B, T, E, K, I, J)
+    dims = (B, T, E, K, I, J)
+    d = _dims_struct(dims)
     mode = _MODES[_scatter_mode]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, (B, T, E, K, I, J), dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, dims, dt))
         stream = _stream_ptr(dev)
-        table = _table_lookup(Ind, (B, T, E, K, I, J), dt, stream)
+        table = _table_state(Ind, dims, dt, stream)[2]
         if table is not None:
             rc = _abi.lib().egs_expert_scatter_forward_table(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
                                                              table.numel(), out.data_ptr(), ws, ws_bytes, d, dt,
@@ -381,10 +409,11 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
     T = grad_X.shape[1]
     grad_Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     grad_W = torch.empty((E, J, I), device=dev, dtype=ct)
-    d = _abi.Dims(B, T, E, K, I, J)
+    dims = (B, T, E, K, I, J)
+    d = _dims_struct(dims)
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
-        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, (B, T, E, K, I, J), dt))
+        keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, dims, dt))
         rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
                                                     grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                     dt, _ind_type_id(Ind), _stream_ptr(dev))

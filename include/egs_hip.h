@@ -210,6 +210,12 @@ int egs_expert_gather_backward_table(const void *X, const void *W, const void *I
                                      int64_t ldx_b, int64_t ldx_t,
                                      int dtype, int ind_dtype, int mode, void *stream);
 
+/* Which capture, if any, `stream` is recording into a HIP graph right now: *id = 0 when it is not capturing, else the
+ * runtime's identifier of that capture (unique per capture in the process).  For bindings that keep a routing table next to
+ * Ind: a table filled by a captured launch holds nothing until the graph is replayed, so it may only serve launches
+ * of the same capture.  No counterpart in the reference.  Returns EGS_ERR_NULL_POINTER / EGS_ERR_HIP. */
+int egs_stream_capture_id(void *stream, unsigned long long *id);
+
 /* ---------------------------------------------------------------------------------------
  * Inference block (new; no single kernel of the reference corresponds to it): the reference's call pattern
  *   out = scatter(act(gather(x, Ind)), Ind, T)          (test_speed.ipynb:73-75)

@@ -22,7 +22,7 @@ TABLE_SHAPES = [
     (2, 256, 32, 32, 128, 64),      # two batch elements of the default shape
     (5, 50, 9, 11, 64, 32),         # ragged K, T, E
     (2, 33, 5, 64, 128, 64),
-    (4, 300, 40, 25, 96, 32),       # 1000 picks per batch element
+    (4, 300, 40, 25, 64, 32),       # 1000 picks per batch element
     (8, 700, 8, 20, 32, 64),        # long T
     (9, 20, 3, 7, 32, 32),
 ]
@@ -147,27 +147,57 @@ def test_a_table_serves_only_the_sizes_and_stream_it_was_built_for():
     assert ATTR not in Ind.__dict__
 
 
-def test_no_table_for_fp32_multi_pass_or_under_capture():
-    for shape, dtype in [((2, 64, 8, 16, 128, 64), torch.float32), ((2, 256, 48, 32, 128, 64), torch.bfloat16)]:
+def test_no_table_for_fp32_multi_pass_or_a_gather_that_cannot_carry_it():
+    for shape, dtype in [((2, 64, 8, 16, 128, 64), torch.float32),       # fp32 scatters sort for themselves
+                         ((2, 256, 48, 32, 128, 64), torch.bfloat16),    # scatter in passes
+                         ((4, 300, 40, 25, 96, 32), torch.bfloat16)]:    # gather forward on the tiled kernel: nothing to ride in
         case = make_case(44, *shape, dtype)
         Ind, _ = chain(case, shape[1])
         assert ATTR not in Ind.__dict__
-    shape = (2, 64, 8, 16, 128, 64)
+
+
+def test_a_table_of_a_captured_launch_serves_that_capture_only():
+    shape = (8, 64, 8, 16, 128, 64)
+    B, T, E, K, I, J = shape
     case = make_case(45, *shape, torch.bfloat16)
+    others = [make_case(46 + i, *shape, torch.bfloat16)["Ind"].to(DEV) for i in range(3)]
     X, Wg, Ws, Y, Ind = (case[k].to(DEV) for k in ("X", "Wg", "Ws", "Y", "Ind"))
-    eager_y = hk.expert_gather_forward_call(X, Wg, Ind.clone(), torch.float32)
-    eager_out = hk.expert_scatter_forward_call(Y, Ws, Ind.clone(), shape[1], torch.float32)
+
+    def eager(ind):
+        hk.set_routing_table_cache(False)
+        r = (hk.expert_gather_forward_call(X, Wg, ind, torch.float32), hk.expert_scatter_forward_call(Y, Ws, ind, T, torch.float32),
+             *hk.expert_gather_backward_call(X, Wg, ind, Y, torch.float32))
+        hk.set_routing_table_cache(True)
+        return r
+
+    hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)       # an eager table exists before the capture starts
+    eager_entry = Ind.__dict__[ATTR]
+    assert eager_entry[0][-1] == 0
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph, stream=side):
+        # the eager table is for another stream and no capture: the captured gather builds its own, the two captured
+        # scatters read it
         gy = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
-        gout = hk.expert_scatter_forward_call(Y, Ws, Ind, shape[1], torch.float32)
-    assert ATTR not in Ind.__dict__, "nothing is left with Ind by a captured call"
-    for _ in range(3):
+        captured_entry = Ind.__dict__[ATTR]
+        assert captured_entry is not eager_entry and captured_entry[0][-1] > 0
+        assert hk._table_lookup(Ind, shape, _abi.BF16, hk._stream_ptr(Ind.device)) is captured_entry[1]
+        gout = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+        gdx, gdw = hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)
+    # after the capture the entry is not used by eager calls (its contents exist only after a replay)
+    assert hk._table_lookup(Ind, shape, _abi.BF16, hk._stream_ptr(Ind.device)) is None
+    for other in [Ind.clone()] + others:
+        Ind.copy_(other)                    # the graph's static input changes between replays
+        want = eager(other)
         graph.replay()
         torch.cuda.synchronize()
-        assert torch.equal(gy, eager_y) and torch.equal(gout, eager_out)
+        for got, ref in zip((gy, gout, gdx, gdw), want):
+            assert torch.equal(got, ref)
+        # eager calls on the same Ind between replays build and use their own table
+        _, mine = chain(case, T, ind=Ind)
+        for got, ref in zip(mine, want):
+            assert torch.equal(got, ref)
 
 
 def test_autograd_chain_uses_and_survives_the_table():
