@@ -92,6 +92,26 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+_pycall = False          # False: not looked for yet; None: not available
+
+
+def pycall():
+    """The CPython module that calls the four launchers of the same library with plain integers (a fraction of the
+    cost of a ctypes call), or None when it has not been built: callers then use ctypes.  Loads the library first,
+    so a missing library is reported the same way on both routes."""
+    global _pycall
+    if _pycall is False:
+        lib()
+        with _lock:
+            if _pycall is False:
+                try:
+                    from . import _egs_pycall as mod
+                    _pycall = mod if mod.abi_version() == ABI_VERSION else None
+                except ImportError:
+                    _pycall = None
+    return _pycall
+
+
 def status_string(status: int) -> str:
     return lib().egs_status_string(status).decode()
 

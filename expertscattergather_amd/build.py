@@ -1,13 +1,16 @@
 """Build recipe of the HIP library (``libegs_hip.so``) for gfx950.
 
 ``python -m expertscattergather_amd.build`` compiles the ``csrc/*.hip`` translation units in-tree with hipcc.
-The library has no torch dependency; the Python side loads it with ctypes.
+The library has no torch dependency; the Python side loads it with ctypes.  A small CPython module
+(``csrc/egs_pycall.c``, built with the host C compiler against the same library) lets the four launchers be
+called with plain integers, which costs a fraction of a ctypes call; without it the Python side uses ctypes.
 """
 from __future__ import annotations
 
 import os
 import subprocess
 import sys
+import sysconfig
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
@@ -37,7 +40,7 @@ def _run(cmd, verbose):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if NOISE not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
+        raise RuntimeError(os.path.basename(cmd[0]) + " failed:\n" + out)
     if verbose and out.strip():
         print(out)
 
@@ -55,7 +58,21 @@ def build(verbose: bool = False, extra_flags=()) -> str:
     with ThreadPoolExecutor(max_workers=len(cmds)) as pool:
         list(pool.map(lambda c: _run(c, verbose), cmds))
     _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH], verbose)
+    build_pycall(verbose)
     return LIB_PATH
+
+
+PYCALL_PATH = os.path.join(HERE, "_egs_pycall" + (sysconfig.get_config_var("EXT_SUFFIX") or ".so"))
+
+
+def build_pycall(verbose: bool = False) -> str:
+    """Compile the CPython module that calls the launchers with integer arguments; it finds libegs_hip.so next to itself."""
+    cc = os.environ.get("CC", "gcc")
+    cmd = [cc, "-O2", "-fPIC", "-shared", "-Wall", "-I", sysconfig.get_paths()["include"],
+           "-I", os.path.join(os.path.dirname(HERE), "include"), os.path.join(CSRC, "egs_pycall.c"),
+           "-L", HERE, "-legs_hip", "-Wl,-rpath,$ORIGIN", "-o", PYCALL_PATH]
+    _run(cmd, verbose)
+    return PYCALL_PATH
 
 
 if __name__ == "__main__":

@@ -320,16 +320,23 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     with _on_device(dev):
         stream = _stream_ptr(dev)
         nb, capture, table = _table_state(Ind, dims, dt, stream)
+        build = None
         if nb and table is None:
             # first sight of these indices: the routing table of the scatters to come is built in this launch
-            table = torch.empty(nb, dtype=torch.uint8, device=dev)
+            build = torch.empty(nb, dtype=torch.uint8, device=dev)
+        fast = _abi.pycall()
+        if fast is not None:
+            rc = fast.gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
+                                     0 if build is None else build.data_ptr(), 0 if build is None else nb,
+                                     B, T, E, K, I, J, ld_b, ld_t, dt, _ind_type_id(Ind), stream or 0)
+        elif build is not None:
             rc = _abi.lib().egs_expert_gather_forward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(),
-                                                            table.data_ptr(), nb, d, ld_b, ld_t, dt, _ind_type_id(Ind), stream)
-            if rc == 0:
-                Ind.__dict__[_TABLE_ATTR] = (_table_key(Ind, dims, dt, stream, capture), table)
+                                                            build.data_ptr(), nb, d, ld_b, ld_t, dt, _ind_type_id(Ind), stream)
         else:
             rc = _abi.lib().egs_expert_gather_forward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), Y.data_ptr(), d,
                                                       ld_b, ld_t, dt, _ind_type_id(Ind), stream)
+        if build is not None and rc == 0:
+            Ind.__dict__[_TABLE_ATTR] = (_table_key(Ind, dims, dt, stream, capture), build)
     if rc:
         _abi.check(rc, "expert_gather_forward_call")
     return Y if res_dtype is ct else Y.to(res_dtype)
@@ -353,7 +360,13 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, dims, dt))
         stream = _stream_ptr(dev)
         table = _table_state(Ind, dims, dt, stream)[2]
-        if table is not None:
+        fast = _abi.pycall()
+        if fast is not None:
+            rc = fast.gather_backward(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), 0 if table is None else table.data_ptr(),
+                                      0 if table is None else table.numel(), grad_output.data_ptr(), grad_X.data_ptr(),
+                                      grad_W.data_ptr(), ws or 0, ws_bytes, B, T, E, K, I, J, ld_b, ld_t, dt,
+                                      _ind_type_id(Ind), mode, stream or 0)
+        elif table is not None:
             rc = _abi.lib().egs_expert_gather_backward_table(X.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
                                                              table.numel(), grad_output.data_ptr(), grad_X.data_ptr(),
                                                              grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t, dt,
@@ -386,7 +399,12 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, dims, dt))
         stream = _stream_ptr(dev)
         table = _table_state(Ind, dims, dt, stream)[2]
-        if table is not None:
+        fast = _abi.pycall()
+        if fast is not None:
+            rc = fast.scatter_forward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), 0 if table is None else table.data_ptr(),
+                                      0 if table is None else table.numel(), out.data_ptr(), ws or 0, ws_bytes,
+                                      B, T, E, K, I, J, dt, _ind_type_id(Ind), mode, stream or 0)
+        elif table is not None:
             rc = _abi.lib().egs_expert_scatter_forward_table(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), table.data_ptr(),
                                                              table.numel(), out.data_ptr(), ws, ws_bytes, d, dt,
                                                              _ind_type_id(Ind), mode, stream)
@@ -414,9 +432,15 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_SCATTER_BACKWARD, 0, dims, dt))
-        rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
-                                                    grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
-                                                    dt, _ind_type_id(Ind), _stream_ptr(dev))
+        fast = _abi.pycall()
+        if fast is not None:
+            rc = fast.scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(), grad_Y.data_ptr(),
+                                       grad_W.data_ptr(), ws or 0, ws_bytes, B, T, E, K, I, J, ld_b, ld_t, dt,
+                                       _ind_type_id(Ind), _stream_ptr(dev) or 0)
+        else:
+            rc = _abi.lib().egs_expert_scatter_backward(Y.data_ptr(), W.data_ptr(), Ind.data_ptr(), grad_X.data_ptr(),
+                                                        grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
+                                                        dt, _ind_type_id(Ind), _stream_ptr(dev))
     del keep
     if rc:
         _abi.check(rc, "expert_scatter_backward_call")

@@ -185,6 +185,32 @@ def test_routing_table_entry_points_validate_without_a_gpu(lib):
     assert gb(p, p, p, t, nb, p, p, p, None, 0, big, *ld, _abi.BF16, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
 
 
+def test_integer_call_module_reaches_the_same_entry_points(lib):
+    fast = _abi.pycall()
+    assert fast is not None, "expertscattergather_amd/_egs_pycall*.so is part of the build"
+    assert fast.abi_version() == _abi.ABI_VERSION
+    p, dims, ld = 0x1000, (64, 256, 32, 32, 128, 64), (256 * 128, 128)
+    d = _abi.Dims(*dims)
+    # the same refusals as through ctypes, before any HIP call
+    assert fast.gather_forward(0, p, p, p, 0, 0, *dims, *ld, _abi.BF16, _abi.IND_I64, 0) == -1 == \
+        lib.egs_expert_gather_forward(None, p, p, p, d, *ld, _abi.BF16, _abi.IND_I64, None)
+    assert fast.gather_forward(p, p, p, p, 0, 0, *dims, *ld, 7, _abi.IND_I64, 0) == _abi.EGS_ERR_BAD_DTYPE
+    assert fast.gather_forward(p, p, p, p, 0x4000, 16, *dims, *ld, _abi.BF16, _abi.IND_I64, 0) == -6       # table too small
+    assert fast.gather_forward(p, p, p, p, 0, 0, 64, 256, -3, 32, 128, 64, *ld, _abi.BF16, _abi.IND_I64, 0) == -2   # negative size
+    assert fast.scatter_forward(p, p, p, 0, 0, p, 0, 0, *dims, _abi.BF16, _abi.IND_I64, 7, 0) == -5          # unknown mode
+    assert fast.scatter_forward(p, p, p, 0, 0, p + 2, 0, 0, *dims, _abi.BF16, _abi.IND_I64, 0, 0) == -6      # general path, no workspace
+    assert fast.gather_backward(p, p, p, 0x4000, 16, p, p, p, 0, 0, *dims, *ld, _abi.BF16, _abi.IND_I64, 0, 0) == -6
+    assert fast.gather_backward(p, p, p, 0, 0, p, p, 0, 0, 0, *dims, *ld, _abi.BF16, _abi.IND_I64, 0, 0) == -1    # null grad_W
+    assert fast.scatter_backward(p, p, p, p, p, 0, 0, 0, *dims, *ld, _abi.BF16, _abi.IND_I64, 0) == -1
+    assert fast.scatter_backward(p, p, p, p, p, p, 0, 0, *dims, 256 * 128, 64, _abi.BF16, _abi.IND_I64, 0) == -10  # token stride < row
+    empty = (0, 256, 32, 32, 128, 64)
+    assert fast.gather_forward(0, 0, 0, 0, 0, 0, *empty, 0, 0, _abi.BF16, _abi.IND_I64, 0) == 0
+    with pytest.raises(TypeError):
+        fast.gather_forward(p, p, p)
+    with pytest.raises(TypeError):
+        fast.scatter_forward(p, p, p, None, 0, p, 0, 0, *dims, _abi.BF16, _abi.IND_I64, 0, 0)
+
+
 def test_planning_functions_survive_arbitrary_sizes(lib):
     # the size queries run the same selection code as the entry points: whatever the sizes, they answer (no
     # division by zero, no overflow into nonsense), in multiples of 256 bytes, and agree with themselves

@@ -751,3 +751,19 @@ def test_concurrent_callers_on_their_own_streams():
         ref = oracle_all(cases[n], shape[1])
         for name in ("Y", "out", "dX", "dWg", "dY", "dWs"):
             assert_close(results[n][name], ref[name], dtype, f"thread {n} {name}")
+
+
+@pytest.mark.parametrize("shape,dtype", [((4, 64, 8, 16, 128, 64), torch.bfloat16), ((2, 300, 4, 200, 256, 192), torch.bfloat16),
+                                         ((3, 40, 6, 100, 24, 16), torch.float32)], ids=["small-bf16", "large-bf16", "general-f32"])
+def test_ctypes_and_integer_call_routes_agree(shape, dtype, monkeypatch):
+    """The launchers reach the library through the integer-call module when it is built and through ctypes otherwise."""
+    from expertscattergather_amd import _abi
+    assert _abi.pycall() is not None
+    case = make_case(77, *shape, dtype)
+    fast = run_all(case, shape[1])
+    monkeypatch.setattr(_abi, "_pycall", None)
+    assert _abi.pycall() is None
+    slow = run_all(case, shape[1])
+    for name in fast:
+        assert torch.equal(fast[name], slow[name]), name
+
