@@ -35,7 +35,7 @@ PROFILES = os.path.join(ROOT, "profiles")
 LAUNCH_KERNELS = {
     "C2": {"expert_gather_forward": "rows_small_kernel", "expert_scatter_forward": "scatter_fused_table_kernel",
            "expert_scatter_backward": "rows_dw_tile_kernel", "expert_gather_backward": "scatter_fused_dwtile_table_kernel"},
-    "C1": {"expert_gather_forward": "rows_small_f32_kernel", "expert_scatter_forward": "scatter_fused_kernel"},
+    "C1": {"expert_gather_forward": "rows_small_f32_kernel", "expert_scatter_forward": "scatter_fused_table_kernel"},
     "C3": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel",
            "expert_scatter_backward": "rows_gemm_dl_kernel + dw_dl_kernel", "expert_gather_backward": "rows_gemm_dl_kernel + segment_sum_kernel + dw_dl_kernel"},
     "C4": {"expert_gather_forward": "rows_gemm_dl_kernel", "expert_scatter_forward": "rows_gemm_dl_kernel + segment_sum_kernel",

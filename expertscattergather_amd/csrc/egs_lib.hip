@@ -395,11 +395,15 @@ int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
 // Two 16-pick row tiles per wavefront and eight wavefronts per workgroup: two wavefronts per SIMD, so that one's waits
 // (row transposition, LDS fragment reads) sit under the other's matrix instructions (default shape 18.4 -> 16.8 us against
 // four row tiles and four wavefronts)
+constexpr int kSmallF32Waves = 8;       // 16 / TQ with TQ = 2 below
+
 template <bool W_NMAJOR, int KS>
 int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t s)
 {
     constexpr int TQ = 2, threads = 64 * (16 / TQ);
-    const size_t lds = rows_small_f32_lds(16 * KS, p.N);
+    static_assert(threads == 64 * kSmallF32Waves, "wavefronts per workgroup");
+    size_t lds = rows_small_f32_lds(16 * KS, p.N);
+    if (p.csr_blocks > 0 && csr_count_lds(p.T, kSmallF32Waves) > lds) lds = csr_count_lds(p.T, kSmallF32Waves);
     switch (p.N / 16) {
     case 1: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 1, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
     case 2: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 2, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
@@ -411,17 +415,28 @@ int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t
 }
 
 // `used` reports whether the shape and operands qualified
+// whether the fp32 small-expert gather takes these sizes and operands
+bool gather_small_f32_takes(const void *X, const void *W, const void *Y, const egs_dims *d, int64_t ldx_b, int64_t ldx_t)
+{
+    const int R = d->I, N = d->J;
+    if (g_force_generic || !(R == 32 || R == 64 || R == 128) || N % 16 != 0 || N < 16 || N > 64 || d->T == 0) return false;
+    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16) || (ldx_b * 4) % 16 || (ldx_t * 4) % 16) return false;
+    const int64_t Me = (int64_t)d->B * d->K;
+    if (Me == 0 || d->E == 0) return false;
+    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + R) * 4;
+    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 4 > kSpan32 || (uint64_t)Me * d->E * N * 4 > kSpan32) return false;
+    const int tiles_per_e = (int)((Me + 255) / 256);
+    return (int64_t)8 * (ceil_div(d->E, 8) + 1) * (tiles_per_e + 8) <= INT32_MAX / 2;
+}
+
+// `build` (optional): the routing table of a later scatter over the same Ind is built by B more workgroups of the launch
 int gather_small_f32(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b, int64_t ldx_t,
-                     int ind_dtype, int w_layout, hipStream_t s, bool &used)
+                     int ind_dtype, int w_layout, hipStream_t s, bool &used, const RoutingTable *build = nullptr)
 {
     used = false;
+    if (!gather_small_f32_takes(X, W, Y, d, ldx_b, ldx_t)) return EGS_OK;
     const int R = d->I, N = d->J;
-    if (g_force_generic || !(R == 32 || R == 64 || R == 128) || N % 16 != 0 || N < 16 || N > 64 || d->T == 0) return EGS_OK;
-    if (!aligned_to(X, 16) || !aligned_to(W, 16) || !aligned_to(Y, 16) || (ldx_b * 4) % 16 || (ldx_t * 4) % 16) return EGS_OK;
     const int64_t Me = (int64_t)d->B * d->K;
-    if (Me == 0 || d->E == 0) return EGS_OK;
-    const uint64_t x_span = ((uint64_t)(d->B - 1) * (uint64_t)ldx_b + (uint64_t)(d->T - 1) * (uint64_t)ldx_t + R) * 4;
-    if (x_span > kSpan32 || (uint64_t)d->E * R * N * 4 > kSpan32 || (uint64_t)Me * d->E * N * 4 > kSpan32) return EGS_OK;
     SmallRowsParams p;
     memset(&p, 0, sizeof(p));
     p.A = (const char *)X; p.W = (const char *)W; p.Ind = Ind; p.C = (char *)Y;
@@ -430,7 +445,8 @@ int gather_small_f32(const void *X, const void *W, const void *Ind, void *Y, con
     p.tiles_per_e = (int)((Me + 255) / 256);
     if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return EGS_OK;
     p.rows_share_xcd = 0;               // W(e) is fetched once per workgroup: experts share an XCD
-    const int blocks = 8 * ceil_div(p.E, 8) * p.tiles_per_e;
+    if (build != nullptr) { p.csr_blocks = d->B; p.seg_off = build->seg; p.perm = build->perm; }
+    const int blocks = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
     used = true;
     const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
     switch (R) {
@@ -780,15 +796,21 @@ struct TableLayout { bool ok; size_t perm_at, bytes; };
 TableLayout routing_table_layout(const egs_dims *d, int act_dtype)
 {
     TableLayout l = {false, 0, 0};
-    if (!(act_dtype == EGS_F16 || act_dtype == EGS_BF16)) return l;
+    if (!(act_dtype == EGS_F16 || act_dtype == EGS_BF16 || act_dtype == EGS_F32)) return l;
     const FusedPlan fp = scatter_fused_plan(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype);
     if (!fp.ok || fp.experts_per_pass != d->E || d->T + 1 > 2048) return l;
     // the table pays only when its build rides in the gather forward's launch (as a launch of its own it costs more than
-    // the two scatters save): the register-resident gather must take these sizes too
-    SmallRowsJob gj;
-    if (!make_gather_small(kStandInPtr, kStandInPtr, kStandInPtr, kStandInPtr, d, (int64_t)d->T * d->I, d->I, act_dtype,
-                           act_dtype, EGS_IND_I32, EGS_W_EIJ, gj))
-        return l;
+    // the two scatters save): the small-expert gather of the type must take these sizes too
+    if (act_dtype == EGS_F32) {
+        if (!gather_small_f32_takes(kStandInPtr, kStandInPtr, kStandInPtr, d, (int64_t)d->T * d->I, d->I) ||
+            csr_count_lds(d->T, kSmallF32Waves) > 64 * 1024)
+            return l;
+    } else {
+        SmallRowsJob gj;
+        if (!make_gather_small(kStandInPtr, kStandInPtr, kStandInPtr, kStandInPtr, d, (int64_t)d->T * d->I, d->I, act_dtype,
+                               act_dtype, EGS_IND_I32, EGS_W_EIJ, gj))
+            return l;
+    }
     l.ok = true;
     l.perm_at = align_up((size_t)d->B * (d->T + 1) * 4, 256);
     l.bytes = l.perm_at + align_up((size_t)d->B * d->E * d->K * 4, 256);
@@ -821,16 +843,14 @@ int gather_gemm_impl(const void *X, const void *W, const void *Ind, void *Y, con
         if (make_gather_small(X, W, Ind, Y, d, ldx_b, ldx_t, act_dtype, w_dtype, ind_dtype, w_layout, j, build))
             return launch_rows_small_job(j, nullptr, nullptr, s);
     }
+    if (w_scale == nullptr && act_dtype == EGS_F32 && w_dtype == EGS_F32) {
+        bool used = false;
+        const int rc = gather_small_f32(X, W, Ind, Y, d, ldx_b, ldx_t, ind_dtype, w_layout, s, used, build);
+        if (used) return rc;
+    }
     if (build != nullptr) {             // no launch for the table to ride in: a launch of its own
         const int rc = launch_routing_table(Ind, ind_dtype, d, build->seg, build->perm, nullptr, nullptr, nullptr, s);
         if (rc != EGS_OK) return rc;
-    }
-    if (w_scale == nullptr) {
-        if (act_dtype == EGS_F32 && w_dtype == EGS_F32) {
-            bool used = false;
-            const int rc = gather_small_f32(X, W, Ind, Y, d, ldx_b, ldx_t, ind_dtype, w_layout, s, used);
-            if (used) return rc;
-        }
     }
     RowsGemmParams p;
     memset(&p, 0, sizeof(p));

@@ -27,7 +27,14 @@ __global__ __launch_bounds__(64 * (16 / TQ)) void rows_small_f32_kernel(SmallRow
     constexpr int PF = KS < 4 ? KS : 4;                                 // slabs of gathered rows in flight
     extern __shared__ __attribute__((aligned(16))) float w_lds[];      // [N][LDW]
     int e, tile;
-    const int bid = (int)blockIdx.x;
+    int bid = (int)blockIdx.x;
+    // routing-table build of a later scatter riding along (csr_blocks = B, or 0): one workgroup per batch element, first in line
+    if (bid < p.csr_blocks) {
+        csr_count_body(reinterpret_cast<int32_t *>(w_lds), bid, bid, (int)threadIdx.x, NTHREADS, p.Ind, p.ind_dtype, p.T,
+                       p.E * p.K, p.seg_off, p.perm, nullptr, nullptr);
+        return;
+    }
+    bid -= p.csr_blocks;
     if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
                          : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;       // uniform per workgroup
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);

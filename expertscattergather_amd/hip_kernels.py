@@ -286,7 +286,7 @@ def _table_nbytes(dims: tuple, dt: int) -> int:
 def _table_state(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
     """(bytes of the table these sizes can use - 0: build and read none now -, capture identifier, the table kept with
     `Ind` if it is valid for this call else None)."""
-    if not _table_cache or dt == _abi.F32 or type(Ind) is not torch.Tensor:
+    if not _table_cache or type(Ind) is not torch.Tensor:
         return 0, 0, None
     nb = _table_nbytes(dims, dt)
     if nb == 0:

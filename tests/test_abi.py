@@ -164,8 +164,9 @@ def test_routing_table_entry_points_validate_without_a_gpu(lib):
     tb = lib.egs_routing_table_bytes
     d = _abi.Dims(64, 256, 32, 32, 128, 64)
     seg, perm = -(-64 * 257 * 4 // 256) * 256, 64 * 32 * 32 * 4
-    assert tb(d, _abi.BF16) == tb(d, _abi.F16) == seg + perm                # [B][T + 1] offsets, then [B][E * K] picks
-    assert tb(d, _abi.F32) == 0                                              # fp32 scatters read no table
+    assert tb(d, _abi.BF16) == tb(d, _abi.F16) == tb(d, _abi.F32) == seg + perm     # [B][T + 1] offsets, then [B][E * K] picks
+    wide = _abi.Dims(64, 256, 32, 32, 128, 128)
+    assert tb(wide, _abi.F32) == 0 and tb(wide, _abi.BF16) == seg + perm     # fp32 one-kernel scatter: reduction 32 / 64 only
     assert tb(_abi.Dims(64, 256, 48, 32, 128, 64), _abi.BF16) == 0           # scatter in passes sorts per pass
     assert tb(_abi.Dims(16, 256, 8, 640, 128, 64), _abi.BF16) == 0           # general path builds its own in the workspace
     assert tb(None, _abi.BF16) == 0 and tb(d, 9) == 0
@@ -174,10 +175,10 @@ def test_routing_table_entry_points_validate_without_a_gpu(lib):
     ld = (256 * 128, 128)
     assert gf(p, p, p, p, t, nb - 1, d, *ld, _abi.BF16, _abi.IND_I64, None) == -6            # table too small
     assert gf(p, p, p, p, t + 16, nb, d, *ld, _abi.BF16, _abi.IND_I64, None) == -7           # not 256-byte aligned
-    assert gf(p, p, p, p, t, nb, d, *ld, _abi.F32, _abi.IND_I64, None) == _abi.EGS_ERR_UNSUPPORTED
+    assert gf(p, p, p, p, t, nb, wide, *ld, _abi.F32, _abi.IND_I64, None) == _abi.EGS_ERR_UNSUPPORTED
     assert gf(None, p, p, p, t, nb, d, *ld, _abi.BF16, _abi.IND_I64, None) == -1
     assert sf(p, p, p, t, nb - 1, p, None, 0, d, _abi.BF16, _abi.IND_I64, 0, None) == -6
-    assert sf(p, p, p, t, nb, p, None, 0, d, _abi.F32, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
+    assert sf(p, p, p, t, nb, p, None, 0, _abi.Dims(64, 256, 32, 32, 256, 64), _abi.F32, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
     assert sf(p, p, p, t, nb, p, None, 0, d, _abi.BF16, _abi.IND_I64, 7, None) == -5          # unknown mode
     assert gb(p, p, p, t, nb - 1, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -6
     assert gb(p, p, p, t + 16, nb, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -7

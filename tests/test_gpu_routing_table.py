@@ -17,7 +17,8 @@ hk.create_kernels()
 DEV = "cuda"
 ATTR = hk._TABLE_ATTR
 
-# 16-bit shapes the one-kernel scatter takes in a single pass (the only consumers of a table)
+# shapes the one-kernel scatter takes in a single pass (the only consumer of a table) in every element type, and whose
+# gather forward runs on a small-expert kernel (the launch that builds it)
 TABLE_SHAPES = [
     (2, 256, 32, 32, 128, 64),      # two batch elements of the default shape
     (5, 50, 9, 11, 64, 32),         # ragged K, T, E
@@ -47,7 +48,7 @@ def chain(case, T, ind=None):
 
 
 @pytest.mark.parametrize("ind_dtype", [torch.int64, torch.int16], ids=["i64", "i16"])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bfloat16", "float16", "float32"])
 @pytest.mark.parametrize("shape", TABLE_SHAPES, ids=lambda s: "x".join(map(str, s)))
 def test_results_do_not_depend_on_the_table(shape, dtype, ind_dtype):
     B, T, E, K, I, J = shape
@@ -63,21 +64,25 @@ def test_results_do_not_depend_on_the_table(shape, dtype, ind_dtype):
     assert_close(tabled[1], O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].to(torch.int64).numpy(), T), dtype, "out")
 
 
-def test_table_is_the_stable_sort_of_the_picks_by_token():
+@pytest.mark.parametrize("dtype,type_id", [(torch.bfloat16, _abi.BF16), (torch.float32, _abi.F32)], ids=["bfloat16", "float32"])
+def test_table_is_the_stable_sort_of_the_picks_by_token(dtype, type_id):
     B, T, E, K, I, J = 5, 50, 9, 11, 64, 32
-    case = make_case(3, B, T, E, K, I, J, torch.bfloat16)
+    case = make_case(3, B, T, E, K, I, J, dtype)
     Ind = case["Ind"].clone()
     Ind[1, 2, 3] = T; Ind[2, 0, 0] = -5         # rejected picks have no place in any token's list
     X, Wg, IndD = case["X"].to(DEV), case["Wg"].to(DEV), Ind.to(DEV)
     d = _abi.Dims(B, T, E, K, I, J)
-    nb = _abi.lib().egs_routing_table_bytes(d, _abi.BF16)
+    nb = _abi.lib().egs_routing_table_bytes(d, type_id)
     assert nb > 0
     table = torch.full((nb,), 0xEE, dtype=torch.uint8, device=DEV)
-    Y = torch.empty(B, E, K, J, dtype=torch.bfloat16, device=DEV)
+    Y = torch.empty(B, E, K, J, dtype=dtype, device=DEV)
     rc = _abi.lib().egs_expert_gather_forward_table(X.data_ptr(), Wg.data_ptr(), IndD.data_ptr(), Y.data_ptr(), table.data_ptr(), nb,
-                                                    d, T * I, I, _abi.BF16, _abi.IND_I64, torch.cuda.current_stream().cuda_stream)
+                                                    d, T * I, I, type_id, _abi.IND_I64, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
+    safe = Ind.clone(); safe[(Ind < 0) | (Ind >= T)] = 0
+    mask = ((Ind >= 0) & (Ind < T)).numpy()[..., None]
+    assert_close(Y, O.gather_forward(np64(case["X"]), np64(case["Wg"]), safe.numpy()) * mask, dtype, "Y of the launch that builds the table")
     words = table.cpu().numpy().view(np.int32)
     perm_at = -(-(B * (T + 1) * 4) // 256) * 256 // 4
     seg = words[:B * (T + 1)].reshape(B, T + 1)
@@ -148,7 +153,7 @@ def test_a_table_serves_only_the_sizes_and_stream_it_was_built_for():
 
 
 def test_no_table_for_fp32_multi_pass_or_a_gather_that_cannot_carry_it():
-    for shape, dtype in [((2, 64, 8, 16, 128, 64), torch.float32),       # fp32 scatters sort for themselves
+    for shape, dtype in [((4, 64, 8, 16, 128, 128), torch.float32),      # fp32 scatter with a reduction of 128: general path
                          ((2, 256, 48, 32, 128, 64), torch.bfloat16),    # scatter in passes
                          ((4, 300, 40, 25, 96, 32), torch.bfloat16)]:    # gather forward on the tiled kernel: nothing to ride in
         case = make_case(44, *shape, dtype)
