@@ -627,7 +627,13 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
 {
     static LdsGrant told_plain, told_dw, told_dwt, told_multi;      // one set per template instantiation
     if constexpr (TT::ES != 2) { dw = nullptr; dwt = nullptr; }     // the small weight gradients exist for 16-bit types only
-    if (p.experts_per_pass < p.E) {
+    if (p.experts_per_pass < p.E && p.tab_seg != nullptr) {
+        static LdsGrant told_multi_tab;
+        const int rc_lds = allow_large_lds((const void *)scatter_fused_multi_table_kernel<TT, W_NMAJOR, KS>, told_multi_tab, lds,
+                                           "hipFuncSetAttribute(scatter_fused_multi_table_kernel)");
+        if (rc_lds != EGS_OK) return rc_lds;
+        hipLaunchKernelGGL((scatter_fused_multi_table_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
+    } else if (p.experts_per_pass < p.E) {
         // several passes over groups of experts: a launch of its own (a weight gradient of the same call follows alone)
         const int rc_lds = allow_large_lds((const void *)scatter_fused_multi_kernel<TT, W_NMAJOR, KS>, told_multi, lds,
                                            "hipFuncSetAttribute(scatter_fused_multi_kernel)");
@@ -724,6 +730,18 @@ FusedPlan scatter_fused_plan(const void *Y, const void *W, const void *Out, cons
     return {true, per_pass, scatter_fused_lds(d->T, (int)NP, per_pass * d->K)};
 }
 
+// whether the one-kernel scatter planned as `fp` can take its routing table from memory: what the kernel's registers stage
+// (one pass: 1024 picks, T + 1 <= 2048 offsets; in passes: 2048 picks, T <= 512, 16-bit types - in fp32 the pass kernel
+// measured slower with the table than sorting for itself: 131 against 128 us for gather + scatter + gather backward at
+// B64 T256 E60 K32 I128 J64)
+bool fused_reads_table(const FusedPlan &fp, const egs_dims *d, int act_dtype)
+{
+    if (!fp.ok) return false;
+    const int64_t NP = (int64_t)d->E * d->K;
+    if (fp.experts_per_pass == d->E) return NP <= 1024 && d->T + 1 <= 2048;
+    return act_dtype != EGS_F32 && NP <= 2048 && d->T <= 512;
+}
+
 bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype)
 {
     return scatter_fused_plan(Y, W, Out, d, act_dtype).ok;
@@ -748,7 +766,7 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.ind_dtype = ind_dtype;
     p.slices = slices;
     p.experts_per_pass = fp.experts_per_pass;
-    if (use != nullptr && fp.experts_per_pass == d->E && NP <= 1024 && d->T + 1 <= 2048) { p.tab_seg = use->seg; p.tab_perm = use->perm; }
+    if (use != nullptr && fused_reads_table(fp, d, act_dtype)) { p.tab_seg = use->seg; p.tab_perm = use->perm; }
     p.perm_at = (int32_t)((int64_t)fp.experts_per_pass * d->K * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
@@ -798,7 +816,7 @@ TableLayout routing_table_layout(const egs_dims *d, int act_dtype)
     TableLayout l = {false, 0, 0};
     if (!(act_dtype == EGS_F16 || act_dtype == EGS_BF16 || act_dtype == EGS_F32)) return l;
     const FusedPlan fp = scatter_fused_plan(kStandInPtr, kStandInPtr, kStandInPtr, d, act_dtype);
-    if (!fp.ok || fp.experts_per_pass != d->E || d->T + 1 > 2048) return l;
+    if (!fused_reads_table(fp, d, act_dtype)) return l;
     // the table pays only when its build rides in the gather forward's launch (as a launch of its own it costs more than
     // the two scatters save): the small-expert gather of the type must take these sizes too
     if (act_dtype == EGS_F32) {

@@ -190,8 +190,9 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     const int EP = MULTI ? p.experts_per_pass : E;
     if constexpr (TABLE) {
         // the table comes from memory: its loads go first, the operands behind them; it is parked in LDS in the places
-        // the sort would have left it while the operands travel (NP <= 1024, T < 2048: checked by the host)
-        constexpr int PV = 1024 / kFusedThreads, SV = 2048 / kFusedThreads;
+        // the sort would have left it while the operands travel (one pass: NP <= 1024, T < 2048; in passes: NP <= 2048,
+        // T <= 512 - checked by the host)
+        constexpr int PV = (MULTI ? 2048 : 1024) / kFusedThreads, SV = (MULTI ? 1024 : 2048) / kFusedThreads;
         const int32_t *gseg = p.tab_seg + (size_t)b * (T + 1), *gperm = p.tab_perm + (size_t)b * NP;
         int32_t pv[PV], sv[SV];
 #pragma unroll
@@ -199,7 +200,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 #pragma unroll
         for (int x = 0; x < SV; ++x) sv[x] = gseg[min(tid + x * kFusedThreads, T)];
 #pragma unroll
-        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, E);
+        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
         int32_t *seg_w = cnt + NWV * T;
 #pragma unroll
         for (int x = 0; x < PV; ++x)
@@ -344,6 +345,13 @@ __global__ __launch_bounds__(kFusedThreads) void scatter_fused_dw_kernel(Scatter
 }
 
 // with the routing table read from memory instead of sorted in the kernel
+template <class TT, bool W_NMAJOR, int KS>
+__global__ __launch_bounds__(kFusedThreads) void scatter_fused_multi_table_kernel(ScatterFusedParams p)
+{
+    extern __shared__ __attribute__((aligned(16))) char smem_fused_multi_table[];
+    scatter_fused_body<TT, W_NMAJOR, KS, true, true>(p, (int)blockIdx.x, smem_fused_multi_table);
+}
+
 template <class TT, bool W_NMAJOR, int KS>
 __global__ __launch_bounds__(kFusedThreads) void scatter_fused_table_kernel(ScatterFusedParams p)
 {

@@ -167,7 +167,8 @@ def test_routing_table_entry_points_validate_without_a_gpu(lib):
     assert tb(d, _abi.BF16) == tb(d, _abi.F16) == tb(d, _abi.F32) == seg + perm     # [B][T + 1] offsets, then [B][E * K] picks
     wide = _abi.Dims(64, 256, 32, 32, 128, 128)
     assert tb(wide, _abi.F32) == 0 and tb(wide, _abi.BF16) == seg + perm     # fp32 one-kernel scatter: reduction 32 / 64 only
-    assert tb(_abi.Dims(64, 256, 48, 32, 128, 64), _abi.BF16) == 0           # scatter in passes sorts per pass
+    assert tb(_abi.Dims(64, 256, 48, 32, 128, 64), _abi.BF16) > 0            # scatter in passes, up to 2048 picks
+    assert tb(_abi.Dims(64, 256, 96, 32, 128, 64), _abi.BF16) == 0           # ... beyond that it sorts for itself
     assert tb(_abi.Dims(16, 256, 8, 640, 128, 64), _abi.BF16) == 0           # general path builds its own in the workspace
     assert tb(None, _abi.BF16) == 0 and tb(d, 9) == 0
     p, t, nb = 0x1000, 0x4000, seg + perm
@@ -182,7 +183,7 @@ def test_routing_table_entry_points_validate_without_a_gpu(lib):
     assert sf(p, p, p, t, nb, p, None, 0, d, _abi.BF16, _abi.IND_I64, 7, None) == -5          # unknown mode
     assert gb(p, p, p, t, nb - 1, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -6
     assert gb(p, p, p, t + 16, nb, p, p, p, None, 0, d, *ld, _abi.BF16, _abi.IND_I64, 0, None) == -7
-    big = _abi.Dims(64, 256, 48, 32, 128, 64)
+    big = _abi.Dims(64, 256, 96, 32, 128, 64)
     assert gb(p, p, p, t, nb, p, p, p, None, 0, big, *ld, _abi.BF16, _abi.IND_I64, 0, None) == _abi.EGS_ERR_UNSUPPORTED
 
 

@@ -26,6 +26,8 @@ TABLE_SHAPES = [
     (4, 300, 40, 25, 64, 32),       # 1000 picks per batch element
     (8, 700, 8, 20, 32, 64),        # long T
     (9, 20, 3, 7, 32, 32),
+    (2, 256, 48, 32, 128, 64),      # 1536 picks: the scatter runs in two passes over groups of experts
+    (4, 100, 20, 100, 64, 32),      # 2000 picks, ragged 32-pick units
 ]
 
 
@@ -58,7 +60,10 @@ def test_results_do_not_depend_on_the_table(shape, dtype, ind_dtype):
     assert ATTR not in ind0.__dict__
     hk.set_routing_table_cache(True)
     ind1, tabled = chain(case, T)
-    assert ATTR in ind1.__dict__, "these sizes have a table: the gather forward must have left one"
+    if dtype is torch.float32 and E * K > 1024:
+        assert ATTR not in ind1.__dict__        # fp32 scatter in passes sorts for itself (measured faster)
+    else:
+        assert ATTR in ind1.__dict__, "these sizes have a table: the gather forward must have left one"
     for a, b, name in zip(plain, tabled, ("Y", "out", "dX", "dWg")):
         assert torch.equal(a, b), f"{name} differs with the table {shape} {dtype}"
     assert_close(tabled[1], O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].to(torch.int64).numpy(), T), dtype, "out")
@@ -154,7 +159,7 @@ def test_a_table_serves_only_the_sizes_and_stream_it_was_built_for():
 
 def test_no_table_for_fp32_multi_pass_or_a_gather_that_cannot_carry_it():
     for shape, dtype in [((4, 64, 8, 16, 128, 128), torch.float32),      # fp32 scatter with a reduction of 128: general path
-                         ((2, 256, 48, 32, 128, 64), torch.bfloat16),    # scatter in passes
+                         ((2, 256, 96, 32, 128, 64), torch.bfloat16),    # scatter in passes over more than 2048 picks
                          ((4, 300, 40, 25, 96, 32), torch.bfloat16)]:    # gather forward on the tiled kernel: nothing to ride in
         case = make_case(44, *shape, dtype)
         Ind, _ = chain(case, shape[1])
