@@ -311,7 +311,8 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
     B, E, K, I, J = _check_shapes(X, W, Ind, None, True)
     res_dtype = X.dtype
     X, ld_b, ld_t = _rows_source(X, ct)
-    W = _dense16(W, ct); Ind = Ind.contiguous()
+    W = _dense16(W, ct)
+    ind_given, Ind = Ind, Ind.contiguous()
     Y = torch.empty((B, E, K, J), device=dev, dtype=ct)
     T = X.shape[1]
     dims = (B, T, E, K, I, J)
@@ -321,7 +322,7 @@ def _gather_forward_impl(X: torch.Tensor, W: torch.Tensor, Ind: torch.Tensor, ou
         stream = _stream_ptr(dev)
         nb, capture, table = _table_state(Ind, dims, dt, stream)
         build = None
-        if nb and table is None:
+        if nb and table is None and Ind is ind_given:      # a contiguous copy made here is gone after this call: nothing to keep a table with
             # first sight of these indices: the routing table of the scatters to come is built in this launch
             build = torch.empty(nb, dtype=torch.uint8, device=dev)
         fast = _abi.pycall()

@@ -234,3 +234,16 @@ def test_autograd_chain_uses_and_survives_the_table():
     again = run()                   # second step with the same Ind object: the table is found, not rebuilt
     for a, b, c in zip(want, got, again):
         assert torch.equal(a, b) and torch.equal(a, c)
+
+
+def test_a_strided_ind_gets_no_table_and_the_same_results():
+    shape = (4, 64, 8, 16, 128, 64)
+    case = make_case(61, *shape, torch.bfloat16)
+    strided = case["Ind"].to(DEV).transpose(1, 2).contiguous().transpose(1, 2)      # [B,E,K] values, K-major memory
+    assert not strided.is_contiguous() and torch.equal(strided.cpu(), case["Ind"])
+    _, got = chain(case, shape[1], ind=strided)
+    assert ATTR not in strided.__dict__, "the launchers work on a contiguous copy that does not outlive the call"
+    hk.set_routing_table_cache(False)
+    _, want = chain(case, shape[1])
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
