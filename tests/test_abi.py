@@ -213,6 +213,23 @@ def test_integer_call_module_reaches_the_same_entry_points(lib):
         fast.scatter_forward(p, p, p, None, 0, p, 0, 0, *dims, _abi.BF16, _abi.IND_I64, 0, 0)
 
 
+def test_header_compiles_as_c99_and_the_library_links_from_c(lib, tmp_path):
+    import shutil
+    import subprocess
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if cc is None:
+        pytest.skip("no C compiler")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.dirname(_abi.LIB_PATH)
+    exe = str(tmp_path / "abi_from_c")
+    build = subprocess.run([cc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(root, "include"),
+                            os.path.join(root, "tests", "c", "abi_from_c.c"), "-L", libdir, "-legs_hip", f"-Wl,-rpath,{libdir}", "-o", exe],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0 and run.stdout.startswith("ok"), run.stdout + run.stderr
+
+
 def test_planning_functions_survive_arbitrary_sizes(lib):
     # the size queries run the same selection code as the entry points: whatever the sizes, they answer (no
     # division by zero, no overflow into nonsense), in multiples of 256 bytes, and agree with themselves
