@@ -146,6 +146,17 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
     issue_n(0);     // does not depend on Ind: overlap with the index fetch below
 
     // ---------------- per-row bookkeeping: where each tile row reads from / writes to
+    // (atomic epilogue: whether two rows of the tile land on the same token is found here, with a bitmap over
+    // (batch element, token) mod kDupBits in the not yet used slab buffer - exact for the rows of one batch element
+    // while T <= kDupBits, on the safe side otherwise)
+    constexpr int kDupBits = 16384;
+    static_assert(EPI != EPI_ATOMIC_F32 || BM * BK * ES >= kDupBits / 8, "bitmap fits the slab buffer");
+    int dup_row = 0;
+    if constexpr (EPI == EPI_ATOMIC_F32) {
+        uint32_t *bitmap = reinterpret_cast<uint32_t *>(smem_m);
+        for (int i = tid; i < kDupBits / 32; i += NT) bitmap[i] = 0u;
+        __syncthreads();
+    }
     const int Me = p.B * p.K;
     if (tid < BM) {
         int m = m0 + tid;
@@ -162,6 +173,11 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
                 if constexpr (EPI == EPI_ATOMIC_F32) {
                     int32_t t = load_token(p.Ind, p.ind_dtype, pick, p.T);
                     co = t < 0 ? -1 : ((int64_t)b * p.T + t) * N;
+                    if (t >= 0) {
+                        const uint32_t key = (uint32_t)((int64_t)b * p.T + t) & (kDupBits - 1);
+                        const uint32_t bit = 1u << (key & 31);
+                        dup_row = (atomicOr(reinterpret_cast<uint32_t *>(smem_m) + (key >> 5), bit) & bit) != 0;
+                    }
                 } else {
                     co = pick * N;
                 }
@@ -170,7 +186,9 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
         a_off[tid] = ao;
         c_off[tid] = co;
     }
-    __syncthreads();
+    bool tile_has_dups = false;
+    if constexpr (EPI == EPI_ATOMIC_F32) tile_has_dups = __syncthreads_or(dup_row) != 0;
+    else __syncthreads();
 
     // ---------------- row-side loader (K-major source rows)
     constexpr int NVM = BM * CH / NT;
@@ -281,19 +299,79 @@ __global__ __launch_bounds__(WM * WN * kWave) void rows_gemm_kernel(RowsGemmPara
             }
         }
     } else {
+        // fp32 atomics on the output.  Rows of the tile that land on the same token (a hot token under a skewed router:
+        // tens of the 128 picks of a tile) are first added up inside the workgroup - LDS atomics into one of kSlots
+        // rows of partial sums - so that the token receives one atomic per column from this tile, not one per pick.
+        // A tile without such rows (the common case, known since the row bookkeeping) goes straight to memory.
         float *cbase = reinterpret_cast<float *>(p.C);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                int64_t co = c_off[wave_m0 + i * 16 + g * 4 + r];
-                if (co < 0) continue;
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    int n = n0 + wave_n0 + j * 16 + a;
-                    if (n < N) unsafeAtomicAdd(cbase + co + n, acc[i][j][r]);
-                }
+        constexpr int kSlots = (BM * BK * ES) / (BN * 4) < 32 ? (BM * BK * ES) / (BN * 4) : 32;
+        static_assert(kSlots >= 8 && BN * BK * ES >= 4 * BM + 16, "bookkeeping of the tile's duplicate rows fits the slab buffers");
+        int16_t *lead = reinterpret_cast<int16_t *>(smem_n);                 // [BM] first row of the tile with the same target
+        int16_t *slot_of = lead + BM;                                        // [BM] slot of a leading row, -1: none
+        int *nslots = reinterpret_cast<int *>(smem_n + 4 * BM);
+        float *dupbuf = reinterpret_cast<float *>(smem_m);                   // [kSlots][BN]
+        if (tile_has_dups) {                                                 // uniform per workgroup
+            __syncthreads();                                                 // the slabs are no longer being read
+            if (tid < BM) { lead[tid] = (int16_t)tid; slot_of[tid] = -1; }
+            if (tid == 0) *nslots = 0;
+            const int64_t my_co = tid < BM ? c_off[tid] : -1;
+            for (int i = tid; i < kSlots * BN; i += NT) dupbuf[i] = 0.f;
+            bool follows = false;
+            if (tid < BM && my_co >= 0) {
+                int l = tid;
+                for (int r = 0; r < BM; ++r)                                 // no early exit: the reads stay independent
+                    if (r < tid && c_off[r] == my_co) l = min(l, r);
+                lead[tid] = (int16_t)l;
+                follows = l != tid;
             }
+            __syncthreads();
+            if (follows) slot_of[lead[tid]] = -2;                            // every writer stores the same value
+            __syncthreads();
+            if (tid < BM && slot_of[tid] == -2) {
+                const int sl = atomicAdd(nslots, 1);
+                slot_of[tid] = (int16_t)(sl < kSlots ? sl : -1);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = wave_m0 + i * 16 + g * 4 + r;
+                    const int l = lead[row], sl = slot_of[l];
+                    if (c_off[row] < 0 || l == row || sl < 0) continue;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) atomicAdd(&dupbuf[sl * BN + wave_n0 + j * 16 + a], acc[i][j][r]);
+                }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = wave_m0 + i * 16 + g * 4 + r;
+                    const int64_t co = c_off[row];
+                    const int l = lead[row], sl = slot_of[l];
+                    if (co < 0 || (l != row && sl >= 0)) continue;           // rejected pick, or folded into its leading row
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        const int nl = wave_n0 + j * 16 + a, n = n0 + nl;
+                        const float extra = (l == row && sl >= 0) ? dupbuf[sl * BN + nl] : 0.f;
+                        if (n < N) unsafeAtomicAdd(cbase + co + n, acc[i][j][r] + extra);
+                    }
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    int64_t co = c_off[wave_m0 + i * 16 + g * 4 + r];
+                    if (co < 0) continue;
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) {
+                        int n = n0 + wave_n0 + j * 16 + a;
+                        if (n < N) unsafeAtomicAdd(cbase + co + n, acc[i][j][r]);
+                    }
+                }
+        }
     }
 }
 

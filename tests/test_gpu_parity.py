@@ -767,3 +767,29 @@ def test_ctypes_and_integer_call_routes_agree(shape, dtype, monkeypatch):
     for name in fast:
         assert torch.equal(fast[name], slow[name]), name
 
+
+
+@pytest.mark.parametrize("shape", [(3, 300, 5, 200, 192, 256),    # 128 x 128 tiles, rows of several batch elements in one tile
+                                   (2, 90, 4, 128, 48, 24),       # 128 x 64 tiles, a tile is exactly the picks of one (b, e)
+                                   (2, 64, 3, 300, 520, 72)],     # more distinct repeated tokens per tile than partial-sum slots
+                         ids=lambda s: "x".join(map(str, s)))
+def test_fp32_atomic_mode_adds_up_repeated_tokens_inside_a_tile(shape):
+    """Skewed routing in the fp32 atomic mode: most picks of an expert land on a handful of tokens, some are rejected."""
+    B, T, E, K, I, J = shape
+    case = make_case(91 + sum(shape), *shape, torch.float32)
+    g = torch.Generator().manual_seed(5)
+    hot = torch.randint(0, T, (B, E, K), generator=g)
+    Ind = case["Ind"].clone()
+    pick_hot = torch.rand(B, E, K, generator=g) < 0.7
+    Ind[pick_hot] = (hot[pick_hot] % 3) * 7 % T             # three hot tokens take 70 % of the picks
+    pairs = torch.rand(B, E, K, generator=g) < 0.5
+    Ind[~pick_hot & pairs] = Ind[~pick_hot & pairs] // 2 * 2 % T   # and many tokens are picked twice or more
+    Ind[0, 0, 0] = -1; Ind[B - 1, E - 1, K - 1] = T
+    bad = (Ind < 0) | (Ind >= T)
+    safe = Ind.clone(); safe[bad] = 0
+    mask = (~bad).numpy()[..., None]
+    got = run_all(dict(case, Ind=Ind), T, mode="atomic")
+    X, Wg, Ws, Y = (np64(case[k]) for k in ("X", "Wg", "Ws", "Y"))
+    assert_close(got["out"], O.scatter_forward(Y * mask, Ws, safe.numpy(), T), torch.float32, "out, skewed atomic")
+    dX, _ = O.gather_backward(X, Wg, safe.numpy(), Y * mask)
+    assert_close(got["dX"], dX, torch.float32, "dX, skewed atomic")
