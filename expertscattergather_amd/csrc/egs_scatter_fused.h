@@ -202,12 +202,14 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 #pragma unroll
         for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
         int32_t *seg_w = cnt + NWV * T;
+        // entries are clamped to what a table of these sizes can hold: whatever a caller hands over (a table of other
+        // indices, memory that was never filled), every loop below ends and every access stays inside the workgroup's rows
 #pragma unroll
         for (int x = 0; x < PV; ++x)
-            if (tid + x * kFusedThreads < NP) perm[tid + x * kFusedThreads] = pv[x];
+            if (tid + x * kFusedThreads < NP) perm[tid + x * kFusedThreads] = min(max(pv[x], 0), NP - 1);
 #pragma unroll
         for (int x = 0; x < SV; ++x)
-            if (tid + x * kFusedThreads <= T) seg_w[tid + x * kFusedThreads] = sv[x];
+            if (tid + x * kFusedThreads <= T) seg_w[tid + x * kFusedThreads] = min(max(sv[x], 0), NP);
     } else {
     csr_count_body(cnt, b, 0, tid, kFusedThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr, [&]() {
 #pragma unroll
@@ -295,7 +297,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
                     for (int x = 0; x < 4; ++x) q[x] = perm[min(cur[i] + x, end[i] - 1)];
 #pragma unroll
                     for (int x = 0; x < 4; ++x) {
-                        const int ql = q[x] < hi ? q[x] - lo : 0;       // picks of later groups: any valid row, not added
+                        const int ql = (q[x] < hi && q[x] >= lo) ? q[x] - lo : 0;   // picks of later groups (or, in a table that is not this Ind's, of earlier ones): any valid row
                         v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)ql * kFusedCols)[cc ^ (ql & 7)];
                     }
                     int n = 0;

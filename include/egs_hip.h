@@ -186,7 +186,8 @@ int egs_gather_gemm_fp8act(const void *X, const void *Wq, const float *w_scale, 
  *   - egs_expert_scatter_forward_table(), egs_expert_gather_backward_table(): the plain entry points with a table that
  *     was filled from the SAME Ind contents and the same sizes; results are bit-identical to the plain entry points.
  *     The table is only read.  A table built from other indices gives wrong sums without any error: the caller owns
- *     that invariant.
+ *     that invariant.  (Its entries are clamped to the ranges a table of these sizes can hold, so even memory that was
+ *     never filled cannot make a kernel run on or touch anything but its own rows.)
  * `table` NULL makes each of these the plain entry point.  A table argument for sizes that have no use for one returns
  * EGS_ERR_UNSUPPORTED; `table` must be 256-byte aligned (EGS_ERR_ALIGNMENT) and at least egs_routing_table_bytes() long
  * (EGS_ERR_WORKSPACE).

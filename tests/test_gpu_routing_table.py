@@ -247,3 +247,25 @@ def test_a_strided_ind_gets_no_table_and_the_same_results():
     _, want = chain(case, shape[1])
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def test_a_table_of_garbage_gives_wrong_sums_but_ends():
+    """The C entry points cannot know whose table they are handed; they must stay inside the workgroup's rows and finish."""
+    for shape in [(4, 64, 8, 16, 128, 64), (2, 256, 48, 32, 128, 64)]:      # one pass, and passes over groups of experts
+        B, T, E, K, I, J = shape
+        case = make_case(71, *shape, torch.bfloat16)
+        Y, Ws, Ind = (case[k].to(DEV) for k in ("Y", "Ws", "Ind"))
+        d = _abi.Dims(*shape)
+        nb = _abi.lib().egs_routing_table_bytes(d, _abi.BF16)
+        assert nb > 0
+        out = torch.empty(B, T, I, dtype=torch.bfloat16, device=DEV)
+        gen = torch.Generator(device="cpu").manual_seed(1)
+        for table in (torch.randint(-2 ** 31, 2 ** 31 - 1, (nb // 4,), generator=gen, dtype=torch.int64).to(torch.int32).to(DEV),
+                      torch.full((nb // 4,), 2 ** 31 - 1, dtype=torch.int32, device=DEV),
+                      torch.zeros(nb // 4, dtype=torch.int32, device=DEV)):
+            rc = _abi.lib().egs_expert_scatter_forward_table(Y.data_ptr(), Ws.data_ptr(), Ind.data_ptr(), table.data_ptr(), nb,
+                                                             out.data_ptr(), None, 0, d, _abi.BF16, _abi.IND_I64, 0,
+                                                             torch.cuda.current_stream().cuda_stream)
+            assert rc == 0
+            torch.cuda.synchronize()
+            assert torch.isfinite(out.float()).all()
