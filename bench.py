@@ -205,6 +205,44 @@ def main():
     use_graph = graph_s is not None and graph_s <= eager_s
     step_s = graph_s if use_graph else eager_s
 
+    # ------------------------------------------------------------------ the same step through the modules and autograd
+    # ExpertScatter(ExpertGather(x, Ind), Ind, T).backward(dOut): the same four launches, issued by PyTorch's autograd
+    # engine (reported beside the step, not as the step: at these sizes it times the engine, not the kernels)
+    autograd_us = None
+    if not fwd_only and not fp8:
+        import expertscattergather_amd as egs
+        gmod = egs.ExpertGather(E, I, J).to(dev, cfg.dtype)
+        smod = egs.ExpertScatter(E, J, I).to(dev, cfg.dtype)
+        with torch.no_grad():
+            gmod.W.copy_(Wg); smod.W.copy_(Ws)
+        xg = X.clone().requires_grad_(True)
+
+        def autograd_step():
+            xg.grad = None; gmod.W.grad = None; smod.W.grad = None
+            smod(gmod(xg, Ind), Ind, T).backward(dOut)
+
+        for _ in range(5):
+            autograd_step()
+        n_auto = max(10, min(args.steps, 100))
+        autograd_us = {"eager": round(time_loop(autograd_step, n_auto) * 1e6, 2), "graph": None}
+        if not args.no_graph:
+            try:
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    for _ in range(3):
+                        autograd_step()
+                torch.cuda.current_stream().wait_stream(side)
+                torch.cuda.synchronize()
+                agraph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(agraph, stream=side):
+                    autograd_step()
+                for _ in range(5):
+                    agraph.replay()
+                autograd_us["graph"] = round(time_loop(agraph.replay, n_auto) * 1e6, 2)
+            except Exception as exc:
+                print(f"bench.py: graph capture of the autograd step failed ({exc})", file=sys.stderr)
+
     # ------------------------------------------------------------------ per-launch timing (HIP events)
     # Every launch of the step through the C ABI, back to back on torch's current stream (the stream the launches are
     # enqueued on), bracketed by HIP events; and once more with the caches flushed before every launch.
@@ -390,6 +428,7 @@ def main():
         "step_tflops": round(chain_flops / step_s * 1e-12, 2),
         "eager_us_per_step": round(eager_s * 1e6, 2),
         "graph_us_per_step": None if graph_s is None else round(graph_s * 1e6, 2),
+        "autograd_us_per_step": autograd_us,
         "routing_table_bytes": int(tab_bytes),
         "launch_us": {k: round(v * 1e6, 2) for k, v in warm.items()},
         "launch_us_cold": None if cold is None else {k: round(v * 1e6, 2) for k, v in cold.items()},
