@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(HERE, "libegs_hip.so")
 # enums of include/egs_hip.h
 EGS_OK = 0
 EGS_ERR_BAD_DTYPE = -3
+EGS_ERR_WORKSPACE = -6
 EGS_ERR_HIP = -8
 EGS_ERR_SCRATCH_LIMIT = -11
 BUILTIN_SCRATCH_BYTES = 16 << 20
@@ -41,6 +42,8 @@ SIGNATURES = {
     "egs_status_string": (ctypes.c_char_p, [_i]),
     "egs_last_hip_error": (ctypes.c_char_p, []),
     "egs_testing_force_generic": (None, [_i]),       # include/egs_hip_testing.h
+    "egs_testing_launch_log_begin": (None, []),
+    "egs_testing_launch_log_end": (_sz, [ctypes.c_char_p, _sz]),
     "egs_workspace_bytes": (_sz, [_i, _i, _dp, _i]),
     "egs_gather_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _dp, _i64, _i64, _i, _i, _i, _i, _vp]),
     "egs_gemm_scatter": (_i, [_vp, _vp, _vp, _vp, _vp, _sz, _dp, _i, _i, _i, _i, _vp]),
@@ -110,6 +113,22 @@ def pycall():
                 except ImportError:
                     _pycall = None
     return _pycall
+
+
+class launch_log:
+    """``with launch_log() as log: ...`` - afterwards ``log.kernels`` lists the kernels the calls of this thread
+    launched inside the block (include/egs_hip_testing.h)."""
+
+    def __enter__(self):
+        self.kernels = []
+        lib().egs_testing_launch_log_begin()
+        return self
+
+    def __exit__(self, *exc):
+        buf = ctypes.create_string_buffer(1024)
+        lib().egs_testing_launch_log_end(buf, len(buf))
+        self.kernels = [k for k in buf.value.decode().split(",") if k]
+        return False
 
 
 def status_string(status: int) -> str:

@@ -28,10 +28,15 @@ constexpr int kMaxDevices = 64;
 struct LdsGrant { std::atomic<uint32_t> bytes[kMaxDevices]; };
 int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *what);
 
+// testing aid (egs_testing_launch_log_begin / _end): while the calling thread keeps a log, the name of every kernel it
+// launches is appended to it
+void note_launch(const char *what);
+
 #define EGS_CHECK_LAUNCH(what)                                         \
     do {                                                               \
         hipError_t err__ = hipGetLastError();                          \
         if (err__ != hipSuccess) return ::egs::host::hip_fail(err__, what); \
+        ::egs::host::note_launch(what);                                \
     } while (0)
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }

@@ -29,6 +29,19 @@ int hip_fail(hipError_t err, const char *what)
 }
 const char *last_hip_error() { return g_hip_error_buf; }
 
+struct LaunchLog { bool on; size_t len; char text[1024]; };
+static thread_local LaunchLog g_launch_log = {false, 0, ""};
+void note_launch(const char *what)
+{
+    LaunchLog &l = g_launch_log;
+    if (!l.on) return;
+    const size_t n = strlen(what);
+    if (l.len + n + 2 > sizeof(l.text)) return;
+    if (l.len > 0) l.text[l.len++] = ',';
+    memcpy(l.text + l.len, what, n + 1);
+    l.len += n;
+}
+
 static std::mutex g_lds_mutex;
 int allow_large_lds(const void *fn, LdsGrant &grant, size_t lds, const char *what)
 {
@@ -386,7 +399,7 @@ int launch_dw_tile_alone(DwTileJob &j, hipStream_t s)
         if (j.act_dtype == EGS_BF16) hipLaunchKernelGGL(dw_tile_kernel<ElemBF16>, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
         else hipLaunchKernelGGL(dw_tile_kernel<ElemF16>, dim3(j.blocks), dim3(kThreads), lds, s, j.q);
     }
-    EGS_CHECK_LAUNCH("dw_tile_kernel");
+    EGS_CHECK_LAUNCH(j.act_dtype == EGS_F32 ? (j.wide ? "dw_tile_wide_f32_kernel" : "dw_tile_kernel") : (j.wide ? "dw_tile_wide_kernel" : "dw_tile_kernel"));
     j.done = true;
     return EGS_OK;
 }
@@ -483,7 +496,7 @@ int launch_rows_small_one(SmallRowsJob &j, SmallDwJob *dw, DwTileJob *dwt, hipSt
         hipLaunchKernelGGL((rows_small_kernel<TT, W_NMAJOR, KS, TN, GATHER, OUT_F32>), dim3(j.blocks), dim3(kThreads),
                            j.lds, s, j.p);
     }
-    EGS_CHECK_LAUNCH("rows_small_kernel");
+    EGS_CHECK_LAUNCH(dw != nullptr ? "rows_dw_small_kernel" : "rows_small_kernel");
     return EGS_OK;
 }
 
@@ -616,7 +629,7 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
     else if (act_dtype == EGS_F16) { if (rows_f32) EGS_SEGSUM(ElemF16, float); else EGS_SEGSUM(ElemF16, uint16_t); }
     else { if (rows_f32) EGS_SEGSUM(ElemBF16, float); else EGS_SEGSUM(ElemBF16, uint16_t); }
 #undef EGS_SEGSUM
-    EGS_CHECK_LAUNCH("segment_sum_kernel");
+    EGS_CHECK_LAUNCH(fuse ? "segsum_dwreduce_kernel" : "segment_sum_kernel");
     if (fuse) reduce->q.S = 1;              // second pass done
     return EGS_OK;
 }
@@ -627,7 +640,9 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
 {
     static LdsGrant told_plain, told_dw, told_dwt, told_multi;      // one set per template instantiation
     if constexpr (TT::ES != 2) { dw = nullptr; dwt = nullptr; }     // the small weight gradients exist for 16-bit types only
+    const char *name = "scatter_fused_kernel";
     if (p.experts_per_pass < p.E && p.tab_seg != nullptr) {
+        name = "scatter_fused_multi_table_kernel";
         static LdsGrant told_multi_tab;
         const int rc_lds = allow_large_lds((const void *)scatter_fused_multi_table_kernel<TT, W_NMAJOR, KS>, told_multi_tab, lds,
                                            "hipFuncSetAttribute(scatter_fused_multi_table_kernel)");
@@ -635,12 +650,14 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
         hipLaunchKernelGGL((scatter_fused_multi_table_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     } else if (p.experts_per_pass < p.E) {
         // several passes over groups of experts: a launch of its own (a weight gradient of the same call follows alone)
+        name = "scatter_fused_multi_kernel";
         const int rc_lds = allow_large_lds((const void *)scatter_fused_multi_kernel<TT, W_NMAJOR, KS>, told_multi, lds,
                                            "hipFuncSetAttribute(scatter_fused_multi_kernel)");
         if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_multi_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     } else if (p.tab_seg != nullptr && dwt != nullptr && !dwt->wide && TT::ES == 2) {
       if constexpr (TT::ES == 2) {
+        name = "scatter_fused_dwtile_table_kernel";
         static LdsGrant told_dwt_tab;
         const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
         const size_t need = lds > tile_lds ? lds : tile_lds;
@@ -652,6 +669,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
         dwt->done = true;
       }
     } else if (p.tab_seg != nullptr && dw == nullptr && (dwt == nullptr || dwt->wide || TT::ES != 2)) {
+        name = "scatter_fused_table_kernel";
         static LdsGrant told_tab;
         const int rc_lds = allow_large_lds((const void *)scatter_fused_table_kernel<TT, W_NMAJOR, KS>, told_tab, lds,
                                            "hipFuncSetAttribute(scatter_fused_table_kernel)");
@@ -659,6 +677,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
         hipLaunchKernelGGL((scatter_fused_table_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     } else if (dwt != nullptr && !dwt->wide) {
       if constexpr (TT::ES == 2) {
+        name = "scatter_fused_dwtile_kernel";
         const size_t tile_lds = dw_tile_lds(kFusedThreads / 64);
         const size_t need = lds > tile_lds ? lds : tile_lds;
         const int rc_lds = allow_large_lds((const void *)scatter_fused_dwtile_kernel<TT, W_NMAJOR, KS>, told_dwt, need,
@@ -670,6 +689,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
       }
     } else if (dw != nullptr) {
       if constexpr (TT::ES == 2) {
+        name = "scatter_fused_dw_kernel";
         const size_t dw_lds = (size_t)kDwSmallLdsBytes * (kFusedThreads / kThreads);       // one 16 KB tile per wavefront
         const size_t need = lds > dw_lds ? lds : dw_lds;
         const int rc_lds = allow_large_lds((const void *)scatter_fused_dw_kernel<TT, W_NMAJOR, KS>, told_dw, need,
@@ -685,7 +705,7 @@ int launch_scatter_fused_one(const ScatterFusedParams &p, size_t lds, int blocks
         if (rc_lds != EGS_OK) return rc_lds;
         hipLaunchKernelGGL((scatter_fused_kernel<TT, W_NMAJOR, KS>), dim3(blocks), dim3(kFusedThreads), lds, s, p);
     }
-    EGS_CHECK_LAUNCH("scatter_fused_kernel");
+    EGS_CHECK_LAUNCH(name);
     return EGS_OK;
 }
 
@@ -1125,6 +1145,23 @@ const char *egs_status_string(int status)
 const char *egs_last_hip_error(void) { return last_hip_error(); }
 
 void egs_testing_force_generic(int on) { g_force_generic.store(on != 0); }
+
+void egs_testing_launch_log_begin(void)
+{
+    g_launch_log.on = true; g_launch_log.len = 0; g_launch_log.text[0] = 0;
+}
+
+size_t egs_testing_launch_log_end(char *buf, size_t n)
+{
+    const size_t len = g_launch_log.len;
+    if (buf != nullptr && n > 0) {
+        const size_t c = len < n - 1 ? len : n - 1;
+        memcpy(buf, g_launch_log.text, c);
+        buf[c] = 0;
+    }
+    g_launch_log.on = false; g_launch_log.len = 0; g_launch_log.text[0] = 0;
+    return len;
+}
 
 size_t egs_workspace_bytes(int op, int mode, const egs_dims *d, int act_dtype)
 {

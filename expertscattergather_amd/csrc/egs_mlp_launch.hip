@@ -86,7 +86,9 @@ int egs_expert_mlp_forward(const void *X, const void *Wg, const void *Ws, const 
     if (!(dtype == EGS_F32 || dtype == EGS_F16 || dtype == EGS_BF16)) return EGS_ERR_BAD_DTYPE;
     if (ind_dtype < EGS_IND_I16 || ind_dtype > EGS_IND_U8) return EGS_ERR_BAD_DTYPE;
     if (activation < EGS_ACT_NONE || activation > EGS_ACT_GELU_TANH) return EGS_ERR_BAD_MODE;
-    if (ldx_t < d->I || ldx_b < (int64_t)d->T * ldx_t) return EGS_ERR_BAD_STRIDE;
+    // the same stride rule as the gather forward: rows must not overlap themselves, batch elements may sit in any
+    // order (a transposed or batch-expanded view passes); the span is checked against the 32-bit offsets in mlp_plan
+    if (ldx_t < d->I || (d->B > 1 && ldx_b < 0)) return EGS_ERR_BAD_STRIDE;
     if ((size_t)d->B * d->T * d->I == 0) return EGS_OK;            // nothing to write
     if (X == nullptr || Out == nullptr) return EGS_ERR_NULL_POINTER;
     if ((size_t)d->E * d->K > 0 && (Wg == nullptr || Ws == nullptr || Ind == nullptr)) return EGS_ERR_NULL_POINTER;

@@ -26,7 +26,7 @@ from . import _abi
 
 __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
-    "set_scatter_mode", "get_scatter_mode", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
+    "set_scatter_mode", "get_scatter_mode", "scatter_mode_scope", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
     "register_reference_namespace", "release_workspaces", "expert_mlp_forward",
     "set_routing_table_cache", "invalidate_routing_table",
 ]
@@ -60,19 +60,46 @@ _MODES = {"deterministic": _abi.SCATTER_DETERMINISTIC, "atomic": _abi.SCATTER_AT
 _scatter_mode = os.environ.get("EGS_SCATTER_MODE", "deterministic").lower()
 if _scatter_mode not in _MODES:
     raise ValueError(f"EGS_SCATTER_MODE must be one of {sorted(_MODES)}, got {_scatter_mode!r}")
+_mode_local = threading.local()         # .override: the mode of the innermost scatter_mode_scope of this thread
 
 
-def set_scatter_mode(mode: str) -> None:
-    """'deterministic' (fixed summation order, bitwise reproducible) or 'atomic' (fp32 atomics)."""
-    global _scatter_mode
+def _check_mode(mode: str) -> str:
     mode = mode.lower()
     if mode not in _MODES:
         raise ValueError(f"scatter mode must be one of {sorted(_MODES)}, got {mode!r}")
-    _scatter_mode = mode
+    return mode
+
+
+def set_scatter_mode(mode: str) -> None:
+    """Process-wide default: 'deterministic' (fixed summation order, bitwise reproducible) or 'atomic' (fp32
+    atomics; 16-bit types: product rows kept in the element type).  A module's ``scatter_mode`` attribute and
+    ``scatter_mode_scope`` take precedence.  A forward call binds the mode in force to its autograd node: the
+    backward of that call runs in the same mode whatever is set by then."""
+    global _scatter_mode
+    _scatter_mode = _check_mode(mode)
 
 
 def get_scatter_mode() -> str:
-    return _scatter_mode
+    """The mode a scatter issued now by this thread would run in."""
+    return getattr(_mode_local, "override", None) or _scatter_mode
+
+
+class scatter_mode_scope:
+    """``with scatter_mode_scope("atomic"): ...`` - the calls this thread makes inside run in that mode
+    (``None``: whatever is in force outside)."""
+
+    def __init__(self, mode):
+        self.mode = None if mode is None else _check_mode(mode)
+
+    def __enter__(self):
+        self.outer = getattr(_mode_local, "override", None)
+        if self.mode is not None:
+            _mode_local.override = self.mode
+        return self
+
+    def __exit__(self, *exc):
+        _mode_local.override = self.outer
+        return False
 
 
 # ------------------------------------------------------------------------------ plumbing
@@ -148,15 +175,18 @@ def _dense16(t: torch.Tensor, ct: torch.dtype) -> torch.Tensor:
 
 _ws_sizes: dict = {}
 _dims_structs: dict = {}
+_cache_lock = threading.Lock()          # the caches are filled without it (a lost insert costs one recomputation); emptying is exclusive
 
 
 def _dims_struct(dims: tuple):
     """The egs_dims structure of a problem, built once per problem (the library only reads it)."""
     d = _dims_structs.get(dims)
     if d is None:
-        if len(_dims_structs) > 4096:
-            _dims_structs.clear()
-        d = _dims_structs[dims] = _abi.Dims(*dims)
+        d = _abi.Dims(*dims)
+        with _cache_lock:
+            if len(_dims_structs) > 4096:
+                _dims_structs.clear()
+            _dims_structs[dims] = d
     return d
 
 
@@ -166,9 +196,11 @@ def _workspace_bytes(op: int, mode: int, dims: tuple, dt: int) -> int:
     key = (op, mode, dims, dt)
     n = _ws_sizes.get(key)
     if n is None:
-        if len(_ws_sizes) > 4096:
-            _ws_sizes.clear()
-        n = _ws_sizes[key] = int(_abi.lib().egs_workspace_bytes(op, mode, _abi.Dims(*dims), dt))
+        n = int(_abi.lib().egs_workspace_bytes(op, mode, _abi.Dims(*dims), dt))
+        with _cache_lock:
+            if len(_ws_sizes) > 4096:
+                _ws_sizes.clear()
+            _ws_sizes[key] = n
     return n
 
 
@@ -286,7 +318,9 @@ def _table_nbytes(dims: tuple, dt: int) -> int:
 def _table_state(Ind: torch.Tensor, dims: tuple, dt: int, stream: int):
     """(bytes of the table these sizes can use - 0: build and read none now -, capture identifier, the table kept with
     `Ind` if it is valid for this call else None)."""
-    if not _table_cache or type(Ind) is not torch.Tensor:
+    # a tensor made under torch.inference_mode() has no version counter (reading it raises, and writes to it are
+    # not recorded): no table is kept with it or read from it
+    if not _table_cache or type(Ind) is not torch.Tensor or Ind.is_inference():
         return 0, 0, None
     nb = _table_nbytes(dims, dt)
     if nb == 0:
@@ -355,7 +389,7 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
     grad_W = torch.empty((E, I, J), device=dev, dtype=ct)
     dims = (B, T, E, K, I, J)
     d = _dims_struct(dims)
-    mode = _MODES[_scatter_mode]
+    mode = _MODES[get_scatter_mode()]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, dims, dt))
@@ -377,7 +411,10 @@ def _gather_backward_impl(X, W, Ind, grad_output, dtype):
                                                        grad_X.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                        dt, _ind_type_id(Ind), mode, stream)
     del keep
-    if rc:
+    if rc == _abi.EGS_ERR_WORKSPACE and not X.is_contiguous():
+        # the scratch is sized for dense operands; a strided view can select kernels that need more: run on a dense copy
+        grad_X, grad_W = _gather_backward_impl(X.contiguous(), W, Ind, grad_output, dtype)
+    elif rc:
         _abi.check(rc, "expert_gather_backward_call")
     return (grad_X if x_dtype is ct else grad_X.to(x_dtype)), (grad_W if w_dtype is ct else grad_W.to(w_dtype))
 
@@ -394,7 +431,7 @@ def _scatter_forward_impl(Y, W, Ind, T, out_dtype):
     out = torch.empty((B, T, I), device=dev, dtype=ct)
     dims = (B, T, E, K, I, J)
     d = _dims_struct(dims)
-    mode = _MODES[_scatter_mode]
+    mode = _MODES[get_scatter_mode()]
     dt = dtype_to_type_id(ct)
     with _on_device(dev):
         keep, ws, ws_bytes = _workspace(dev, _workspace_bytes(_abi.OP_GEMM_SCATTER, mode, dims, dt))
@@ -443,7 +480,9 @@ def _scatter_backward_impl(Y, W, Ind, grad_X, dtype):
                                                         grad_Y.data_ptr(), grad_W.data_ptr(), ws, ws_bytes, d, ld_b, ld_t,
                                                         dt, _ind_type_id(Ind), _stream_ptr(dev))
     del keep
-    if rc:
+    if rc == _abi.EGS_ERR_WORKSPACE and not grad_X.is_contiguous():
+        grad_Y, grad_W = _scatter_backward_impl(Y, W, Ind, grad_X.contiguous(), dtype)    # see _gather_backward_impl
+    elif rc:
         _abi.check(rc, "expert_scatter_backward_call")
     return (grad_Y if y_dtype is ct else grad_Y.to(y_dtype)), (grad_W if w_dtype is ct else grad_W.to(w_dtype))
 
@@ -507,10 +546,12 @@ def _register_ops(ns: str) -> None:
         X, W, Ind, out_dtype = inputs
         ctx.save_for_backward(X, W, Ind)
         ctx.out_dtype = out_dtype
+        ctx.scatter_mode = _mode_to_bind()
 
     def gather_backward(ctx, grad_output):
         X, W, Ind = ctx.saved_tensors
-        grad_X, grad_W = ops.expert_gather_backward_call_fn(X, W, Ind, grad_output, ctx.out_dtype)
+        with scatter_mode_scope(ctx.scatter_mode):      # grad_X is a scatter: in the mode the forward was called in
+            grad_X, grad_W = ops.expert_gather_backward_call_fn(X, W, Ind, grad_output, ctx.out_dtype)
         return grad_X, grad_W, None, None
 
     def scatter_setup(ctx, inputs, output):
@@ -589,6 +630,12 @@ def register_reference_namespace(ns: str = "mylib") -> None:
 
 
 # ------------------------------------------------------------------------------ autograd Functions
+def _mode_to_bind():
+    """The scatter mode a forward call hands to its backward; None while torch.compile is tracing (thread-local state
+    is not traced: the compiled backward then runs in the mode in force when it is called)."""
+    return None if torch.compiler.is_compiling() else get_scatter_mode()
+
+
 class ExpertGatherFunction(torch.autograd.Function):
     """Y[b,e,k,j] = sum_i X[b, Ind[b,e,k], i] * W[e,i,j]   (reference egs/triton_kernels.py:581-608)."""
 
@@ -597,12 +644,17 @@ class ExpertGatherFunction(torch.autograd.Function):
         create_kernels()
         ctx.save_for_backward(X, W, Ind)
         ctx.dtype = out_type
+        ctx.scatter_mode = _mode_to_bind()
         return expert_gather_forward_call(X, W, Ind, out_type)
 
     @staticmethod
     def backward(ctx, grad_output: torch.Tensor):
         X, W, Ind = ctx.saved_tensors
-        grad_X, grad_W = expert_gather_backward_call(X, W, Ind, grad_output, ctx.dtype)
+        if ctx.scatter_mode is None:
+            grad_X, grad_W = expert_gather_backward_call(X, W, Ind, grad_output, ctx.dtype)
+        else:
+            with scatter_mode_scope(ctx.scatter_mode):      # grad_X is a scatter: in the mode the forward was called in
+                grad_X, grad_W = expert_gather_backward_call(X, W, Ind, grad_output, ctx.dtype)
         return grad_X, grad_W, None, None
 
 

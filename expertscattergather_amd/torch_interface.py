@@ -8,14 +8,19 @@ import math
 import torch
 from torch import nn
 
-from .hip_kernels import ExpertGatherFunction, ExpertScatterFunction, create_kernels
+from .hip_kernels import ExpertGatherFunction, ExpertScatterFunction, create_kernels, scatter_mode_scope
 
 
 class ExpertGather(nn.Module):
     """Gathers K tokens per (batch, expert) and applies that expert's [I,J] weight.
 
     Reference: egs/torch_interface.py:11-63.  ``W`` is [E,I,J]; the optional ``bias`` is
-    [E,1,J] and is added to every picked row of its expert."""
+    [E,1,J] and is added to every picked row of its expert.
+
+    ``scatter_mode`` (attribute, default ``None`` = the process-wide setting of ``hip_kernels.set_scatter_mode`` /
+    ``EGS_SCATTER_MODE``): "deterministic" or "atomic" for the scatter in this module's backward (grad of ``x``)."""
+
+    scatter_mode = None
 
     def __init__(self, E: int, I: int, J: int, bias: bool = False):
         super().__init__()
@@ -36,7 +41,11 @@ class ExpertGather(nn.Module):
 
     def forward(self, x: torch.Tensor, Ind: torch.Tensor):
         """x: [B,T,I];  Ind: integers in [0,T) of shape [B,E,K]  ->  [B,E,K,J]."""
-        y = ExpertGatherFunction.apply(x, self.W, Ind)
+        if self.scatter_mode is None:
+            y = ExpertGatherFunction.apply(x, self.W, Ind)
+        else:
+            with scatter_mode_scope(self.scatter_mode):     # bound to the autograd node: the backward runs in it too
+                y = ExpertGatherFunction.apply(x, self.W, Ind)
         if self.bias is not None:
             y = y + self.bias
         return y
@@ -49,7 +58,12 @@ class ExpertScatter(nn.Module):
     """Applies each expert's [J,I] weight to its K rows and adds them back onto their tokens.
 
     Reference: egs/torch_interface.py:66-119.  ``W`` is [E,J,I]; the optional ``bias`` is
-    [E,1,I] and every pick of expert e adds bias[e] to the token it lands on."""
+    [E,1,I] and every pick of expert e adds bias[e] to the token it lands on.
+
+    ``scatter_mode`` (attribute, default ``None`` = the process-wide setting of ``hip_kernels.set_scatter_mode`` /
+    ``EGS_SCATTER_MODE``): "deterministic" or "atomic" for this module's forward."""
+
+    scatter_mode = None
 
     def __init__(self, E: int, J: int, I: int, bias: bool = False):
         super().__init__()
@@ -70,7 +84,11 @@ class ExpertScatter(nn.Module):
 
     def forward(self, Y: torch.Tensor, Ind: torch.Tensor, T: int):
         """Y: [B,E,K,J];  Ind: [B,E,K] in [0,T);  T: output sequence length  ->  [B,T,I]."""
-        y = ExpertScatterFunction.apply(Y, self.W, Ind, T)
+        if self.scatter_mode is None:
+            y = ExpertScatterFunction.apply(Y, self.W, Ind, T)
+        else:
+            with scatter_mode_scope(self.scatter_mode):
+                y = ExpertScatterFunction.apply(Y, self.W, Ind, T)
         if self.bias is not None and T > 0 and Ind.numel() > 0:
             # picks[b,t,e] = how many times expert e selected token t; each adds bias[e]
             # (a pick outside [0,T) contributes nothing, as in the kernels: it is routed to slot 0 with weight 0)

@@ -6,6 +6,8 @@
 #ifndef EGS_HIP_TESTING_H
 #define EGS_HIP_TESTING_H
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -15,6 +17,13 @@ extern "C" {
  * the oracle on the same inputs (both must stay within the same tolerances).  Process-wide; the
  * test-suite sets and clears it around single-threaded test cases. */
 void egs_testing_force_generic(int on);
+
+/* Which kernels did a call select?  _begin starts (and empties) a log kept for the calling thread; every kernel the
+ * thread then launches through the library appends its name; _end copies the comma-separated names into `buf` (at most
+ * n - 1 characters and a terminating 0), stops the log and returns the length of the full text.  Used by the benchmark
+ * to name the kernels behind the launches it times, and by tests that assert which path a shape took. */
+void egs_testing_launch_log_begin(void);
+size_t egs_testing_launch_log_end(char *buf, size_t n);
 
 #ifdef __cplusplus
 }

@@ -793,3 +793,110 @@ def test_fp32_atomic_mode_adds_up_repeated_tokens_inside_a_tile(shape):
     assert_close(got["out"], O.scatter_forward(Y * mask, Ws, safe.numpy(), T), torch.float32, "out, skewed atomic")
     dX, _ = O.gather_backward(X, Wg, safe.numpy(), Y * mask)
     assert_close(got["dX"], dX, torch.float32, "dX, skewed atomic")
+
+
+def test_tensors_made_under_inference_mode():
+    """Tensors created under torch.inference_mode() carry no version counter: the forward launchers and the inference
+    block must neither read one nor keep a routing table with such an Ind."""
+    B, T, E, K, I, J = 8, 256, 32, 32, 128, 64          # the default shape's kernels (its routing table applies)
+    dtype = torch.bfloat16
+    case = make_case(53, B, T, E, K, I, J, dtype)
+    with torch.inference_mode():
+        X, Wg, Ws, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Ind"))
+        assert Ind.is_inference()
+        Y = hk.expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        out = hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32)
+        blk = hk.expert_mlp_forward(X, Wg, Ws, Ind, "relu")
+        composed = hk.expert_mlp_forward(X, Wg, Ws, Ind, "gelu")        # E * K / 32 > 16: the two launchers with torch's gelu
+        mods = egs.ExpertScatter(E, J, I).to(DEV, dtype)(egs.ExpertGather(E, I, J).to(DEV, dtype)(X, Ind), Ind, T)
+        torch.cuda.synchronize()
+    assert hk._TABLE_ATTR not in Ind.__dict__
+    assert mods.shape == (B, T, I)
+    Xn, Wgn, Wsn, Indn = np64(case["X"]), np64(case["Wg"]), np64(case["Ws"]), case["Ind"].numpy()
+    assert_close(Y, O.gather_forward(Xn, Wgn, Indn), dtype, "Y under inference_mode")
+    assert_close(out, O.scatter_forward(np64(Y), Wsn, Indn, T), dtype, "out under inference_mode")
+    assert_close(blk, _mlp_oracle(case, T, "relu", dtype), dtype, "inference block under inference_mode")
+    assert_close(composed, _mlp_oracle(case, T, "gelu", dtype, stored_y=True), dtype, "composed block under inference_mode")
+
+
+def test_inference_block_takes_the_views_the_gather_takes():
+    """A batch/token-transposed X and a batch-expanded X (batch stride 0) go through the block like through the gather."""
+    B, T, E, K, I, J = 8, 64, 8, 16, 128, 64
+    dtype = torch.bfloat16
+    case = make_case(59, B, T, E, K, I, J, dtype)
+    Wg, Ws, Ind = (dev(case[k]) for k in ("Wg", "Ws", "Ind"))
+    Xt = dev(case["X"]).transpose(0, 1).contiguous().transpose(0, 1)      # [B,T,I] view with strides (I, B*I, 1)
+    assert not Xt.is_contiguous() and Xt.stride(0) < Xt.stride(1)
+    ref = _mlp_oracle(case, T, "relu", dtype)
+    assert_close(hk.expert_mlp_forward(Xt, Wg, Ws, Ind, "relu", force_block=True), ref, dtype, "block, transposed X")
+    x0 = dev(case["X"][:1])
+    Xe = x0.expand(B, T, I)                                               # batch stride 0
+    assert Xe.stride(0) == 0
+    case_e = dict(case, X=case["X"][:1].expand(B, T, I).contiguous())
+    assert_close(hk.expert_mlp_forward(Xe, Wg, Ws, Ind, "relu", force_block=True), _mlp_oracle(case_e, T, "relu", dtype), dtype,
+                 "block, expanded X")
+    assert_close(hk.expert_gather_forward_call(Xe, Wg, Ind, torch.float32),
+                 O.gather_forward(np64(case_e["X"]), np64(case["Wg"]), case["Ind"].numpy()), dtype, "gather, expanded X")
+
+
+def test_module_scatter_mode_overrides_the_global_and_is_bound_at_forward():
+    """`module.scatter_mode` wins over the process-wide mode, and a backward issued after the process-wide mode has been
+    switched still runs in the mode its forward was called in (16-bit types beyond the one-kernel scatter: the two modes
+    differ in the precision of the product rows, so their results differ in a few last bits)."""
+    B, T, E, K, I, J = 2, 300, 4, 200, 256, 192
+    dtype = torch.bfloat16
+    case = make_case(61, B, T, E, K, I, J, dtype)
+    Y, Ws, Ind, dOut, X, Wg = (dev(case[k]) for k in ("Y", "Ws", "Ind", "dOut", "X", "Wg"))
+    ref = {}
+    for mode in ("deterministic", "atomic"):
+        hk.set_scatter_mode(mode)
+        try:
+            ref[mode] = (hk.expert_scatter_forward_call(Y, Ws, Ind, T, torch.float32),
+                         hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)[0])
+        finally:
+            hk.set_scatter_mode("deterministic")
+    assert not torch.equal(ref["deterministic"][0], ref["atomic"][0])   # otherwise the test below proves nothing
+    smod = egs.ExpertScatter(E, J, I).to(DEV, dtype)
+    gmod = egs.ExpertGather(E, I, J).to(DEV, dtype)
+    with torch.no_grad():
+        smod.W.copy_(Ws); gmod.W.copy_(Wg)
+    smod.scatter_mode = "atomic"
+    assert torch.equal(smod(Y, Ind, T), ref["atomic"][0])
+    smod.scatter_mode = None
+    assert torch.equal(smod(Y, Ind, T), ref["deterministic"][0])
+    # the gather's backward scatters: mode bound when the forward ran
+    gmod.scatter_mode = "atomic"
+    x = X.clone().requires_grad_(True)
+    y = gmod(x, Ind)
+    gmod.scatter_mode = None
+    y.backward(Y)
+    assert torch.equal(x.grad, ref["atomic"][1])
+    x = X.clone().requires_grad_(True)
+    y = gmod(x, Ind)                       # deterministic now
+    hk.set_scatter_mode("atomic")
+    try:
+        y.backward(Y)
+    finally:
+        hk.set_scatter_mode("deterministic")
+    assert torch.equal(x.grad, ref["deterministic"][1])
+
+
+def test_fp32_atomic_mode_at_zipf_sizes():
+    """fp32 atomic mode at the sizes of the Zipf-routed configuration (two batch elements): a quarter of the picks on one
+    token, far more distinct repeated tokens per 128-row tile than the in-tile pre-reduction has slots for."""
+    from expertscattergather_amd import workloads as wl
+    cfg = wl.CONFIGS["C4"]
+    B, T, E, K, I, J = 2, cfg.T, cfg.E, cfg.K, cfg.I, cfg.J
+    inp = wl.make_inputs(cfg, dims=(B, T, E, K, I, J))
+    Y = torch.randn(B, E, K, J, generator=torch.Generator().manual_seed(7))
+    Ws = inp["Ws"].float()
+    Ind = inp["Ind"]
+    counts = torch.bincount(Ind[0].reshape(-1), minlength=T)
+    assert counts.max() > 0.15 * E * K
+    hk.set_scatter_mode("atomic")
+    try:
+        out = hk.expert_scatter_forward_call(dev(Y), dev(Ws), dev(Ind), T, torch.float32)
+        torch.cuda.synchronize()
+    finally:
+        hk.set_scatter_mode("deterministic")
+    assert_close(out, O.scatter_forward(np64(Y), np64(Ws), Ind.numpy(), T), torch.float32, "fp32 atomic, Zipf sizes")

@@ -76,6 +76,49 @@ def test_scatter_mode_switch():
     hk.set_scatter_mode(keep)
 
 
+def test_scatter_mode_scope_and_module_attribute():
+    """The mode in force is: innermost scope of the thread, else the process-wide setting; a module's
+    `scatter_mode` attribute is such a scope around its call, and other threads do not see it."""
+    import threading
+    import expertscattergather_amd as egs
+    keep = hk.get_scatter_mode()
+    try:
+        hk.set_scatter_mode("deterministic")
+        with hk.scatter_mode_scope("atomic"):
+            assert hk.get_scatter_mode() == "atomic"
+            with hk.scatter_mode_scope(None):
+                assert hk.get_scatter_mode() == "atomic"
+            with hk.scatter_mode_scope("Deterministic"):
+                assert hk.get_scatter_mode() == "deterministic"
+            assert hk.get_scatter_mode() == "atomic"
+            seen = []
+            th = threading.Thread(target=lambda: seen.append(hk.get_scatter_mode()))
+            th.start(); th.join()
+            assert seen == ["deterministic"]
+        assert hk.get_scatter_mode() == "deterministic"
+        with pytest.raises(ValueError):
+            hk.scatter_mode_scope("fastest")
+        g, s = egs.ExpertGather(2, 8, 4), egs.ExpertScatter(2, 4, 8)
+        assert g.scatter_mode is None and s.scatter_mode is None
+        # the modules hand the mode in force to their Functions: record it instead of launching
+        seen = []
+        orig_g, orig_s = hk.expert_gather_forward_call, hk.expert_scatter_forward_call
+        hk.expert_gather_forward_call = lambda X, W, Ind, dt: (seen.append(hk.get_scatter_mode()), torch.zeros(1, 2, 3, 4))[1]
+        hk.expert_scatter_forward_call = lambda Y, W, Ind, T, dt: (seen.append(hk.get_scatter_mode()), torch.zeros(1, T, 8))[1]
+        try:
+            Ind = torch.zeros(1, 2, 3, dtype=torch.int64)
+            g.scatter_mode = "atomic"
+            g(torch.zeros(1, 5, 8), Ind)
+            s(torch.zeros(1, 2, 3, 4), Ind, 5)
+            s.scatter_mode = "atomic"
+            s(torch.zeros(1, 2, 3, 4), Ind, 5)
+        finally:
+            hk.expert_gather_forward_call, hk.expert_scatter_forward_call = orig_g, orig_s
+        assert seen == ["atomic", "deterministic", "atomic"] and hk.get_scatter_mode() == "deterministic"
+    finally:
+        hk.set_scatter_mode(keep)
+
+
 def test_workloads_follow_the_benchmark_configurations():
     assert wl.CONFIGS["C2"].dims == (64, 256, 32, 32, 128, 64)
     assert wl.algorithmic_bytes(wl.CONFIGS["C2"].dims, 2) == 13631488
