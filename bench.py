@@ -67,7 +67,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", default="C2", help="workload (C2 = the metric's configuration)")
-    ap.add_argument("--mode", default=None, choices=["deterministic", "atomic"], help="scatter mode (default: env / deterministic)")
+    ap.add_argument("--mode", default=None, choices=["deterministic", "atomic", "compact"], help="scatter mode (default: env / deterministic)")
     ap.add_argument("--fp8-act", action="store_true",
                     help="C5 only: quantise the activations per row to e4m3 and multiply on the fp8 matrix instruction")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches only, no HIP graph replays")
@@ -235,7 +235,7 @@ class Workload:
         out = torch.empty(B, T, I, device=dev, dtype=cfg.dtype)
         dYb, dXb = torch.empty_like(Y), torch.empty(B, T, I, device=dev, dtype=cfg.dtype)
         dWg_b, dWs_b = torch.empty(E, I, J, device=dev, dtype=cfg.dtype), torch.empty(E, J, I, device=dev, dtype=cfg.dtype)
-        mode = 0 if self.mode == "deterministic" else 1
+        mode = hk._MODES[self.mode]
         ws_bytes = max(lib.egs_workspace_bytes(_abi.OP_GATHER_BACKWARD, mode, d, dt), lib.egs_workspace_bytes(_abi.OP_DW, mode, d, dt), 256)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         f8ws_bytes = lib.egs_gather_gemm_fp8act_workspace_bytes(d) if fp8_act else 0
@@ -366,6 +366,8 @@ def side_config(name, mode, traffic, fp8_act=False):
     dom = max(warm, key=warm.get)
     roofs = {lname: w.roofline_of(lname, warm[lname], None, traffic) for lname in launches}
     res = {"workload": f"{w.cfg.name}: B{B} T{T} E{E} K{K} I{I} J{J} {w.cfg.what}", "scatter_mode": mode,
+           "scatter_workspace_bytes": int(w.abi.lib().egs_workspace_bytes(w.abi.OP_GEMM_SCATTER, w.hk._MODES[mode], w.abi.Dims(*w.dims),
+                                                                             w.hk.dtype_to_type_id(w.cfg.dtype))),
            "dtype": ("fp8 x fp8" if fp8_act else w.dtype_name + (" (fp8 e4m3 weights)" if w.fp8 else "")),
            "step_us": round(step_us, 1), "launch": how,
            "step_hbm_frac": round(w.chain_bytes / (step_us * 1e-6) * 1e-9 / HBM_PEAK_GBPS, 4),
@@ -522,7 +524,8 @@ def main():
     configs = None
     if headline and not args.no_configs:
         configs = {}
-        for name, m in (("C1", "deterministic"), ("C3", "deterministic"), ("C4", "deterministic"), ("C4", "atomic"), ("C5", "deterministic")):
+        for name, m in (("C1", "deterministic"), ("C3", "deterministic"), ("C4", "deterministic"), ("C4", "atomic"), ("C4", "compact"),
+                        ("C5", "deterministic")):
             t0 = time.perf_counter()
             try:
                 configs[name if name != "C4" else f"C4-{m}"] = dict(side_config(name, m, traffic), bench_s=round(time.perf_counter() - t0, 1))

@@ -22,7 +22,7 @@ BUILTIN_SCRATCH_BYTES = 16 << 20
 F32, F16, BF16, FP8_E4M3 = 0, 1, 2, 3
 IND_I16, IND_I32, IND_I64, IND_U8 = 0, 1, 2, 3
 W_EIJ, W_EJI = 0, 1
-SCATTER_DETERMINISTIC, SCATTER_ATOMIC = 0, 1
+SCATTER_DETERMINISTIC, SCATTER_ATOMIC, SCATTER_COMPACT = 0, 1, 2
 OP_GATHER_GEMM, OP_GEMM_SCATTER, OP_DW, OP_GATHER_BACKWARD, OP_SCATTER_BACKWARD = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_SILU, ACT_GELU_TANH = 0, 1, 2, 3, 4
 EGS_ERR_UNSUPPORTED = -9

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libegs_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["egs_lib.hip", "egs_rows_launch.hip", "egs_dw_launch.hip", "egs_f8_launch.hip", "egs_mlp_launch.hip"]
+SOURCES = ["egs_lib.hip", "egs_rows_launch.hip", "egs_dw_launch.hip", "egs_f8_launch.hip", "egs_mlp_launch.hip", "egs_pass_launch.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

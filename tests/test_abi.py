@@ -53,7 +53,7 @@ def test_enums_match_header():
                         ("EGS_FP8_E4M3", _abi.FP8_E4M3), ("EGS_IND_I16", _abi.IND_I16), ("EGS_IND_I32", _abi.IND_I32),
                         ("EGS_IND_I64", _abi.IND_I64), ("EGS_IND_U8", _abi.IND_U8), ("EGS_W_EIJ", _abi.W_EIJ),
                         ("EGS_W_EJI", _abi.W_EJI), ("EGS_SCATTER_DETERMINISTIC", _abi.SCATTER_DETERMINISTIC),
-                        ("EGS_SCATTER_ATOMIC", _abi.SCATTER_ATOMIC), ("EGS_OP_GATHER_BACKWARD", _abi.OP_GATHER_BACKWARD),
+                        ("EGS_SCATTER_ATOMIC", _abi.SCATTER_ATOMIC), ("EGS_SCATTER_COMPACT", _abi.SCATTER_COMPACT), ("EGS_OP_GATHER_BACKWARD", _abi.OP_GATHER_BACKWARD),
                         ("EGS_OP_SCATTER_BACKWARD", _abi.OP_SCATTER_BACKWARD), ("EGS_ERR_HIP", _abi.EGS_ERR_HIP)):
         m = re.search(rf"\b{name}\s*=\s*(-?\d+)", text)
         assert m and int(m.group(1)) == value, name
@@ -125,6 +125,13 @@ def test_workspace_sizes_are_consistent(lib):
     assert wb(_abi.OP_SCATTER_BACKWARD, 0, d, _abi.BF16) == dw
     assert wb(_abi.OP_GEMM_SCATTER, 1, d, _abi.F32) == 0                      # fp32 atomic mode adds into the output
     assert det % 256 == 0 and dw % 256 == 0
+    # compact mode (16-bit types, reduction 32 / 64 / 128, T <= 1024): the routing table and nothing else
+    compact = wb(_abi.OP_GEMM_SCATTER, _abi.SCATTER_COMPACT, d, _abi.BF16)
+    table = 16 * (256 + 1) * 4 + 2 * 16 * 8 * 640 * 4
+    assert table <= compact <= table + 3 * 256 and compact < det // 50
+    assert wb(_abi.OP_GEMM_SCATTER, _abi.SCATTER_COMPACT, d, _abi.F32) == wb(_abi.OP_GEMM_SCATTER, 0, d, _abi.F32)   # fp32: as deterministic
+    assert wb(_abi.OP_GEMM_SCATTER, _abi.SCATTER_COMPACT, _abi.Dims(8, 4096, 128, 256, 1024, 256), _abi.BF16) == \
+        wb(_abi.OP_GEMM_SCATTER, 0, _abi.Dims(8, 4096, 128, 256, 1024, 256), _abi.BF16)                              # T > 1024
     assert wb(99, 0, d, 2) == 0 and wb(_abi.OP_DW, 0, d, 9) == 0
     # an entry point checks the workspace against the kernels its actual operands select: an output that is not
     # 16-byte aligned cannot take the one-kernel scatter and is refused without the general path's workspace

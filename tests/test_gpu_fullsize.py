@@ -117,6 +117,37 @@ def test_c3_long_sequence_bf16():
 
 def test_c4_zipf_routing_both_modes():
     check_large("C4", ["deterministic", "atomic"])
+    # compact mode: the configuration's scatters (forward, and dX in the gather's backward) run in one kernel each, product
+    # rows in LDS and a workspace of the routing table only; the other modes go through product rows in the workspace
+    from expertscattergather_amd import _abi
+    cfg, inp, g = gpu_inputs("C4")
+    B, T, E, K, I, J = cfg.dims
+    d = _abi.Dims(*cfg.dims)
+    ws = {m: _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, v, d, _abi.BF16) for m, v in
+          (("deterministic", 0), ("atomic", 1), ("compact", 2))}
+    assert ws["compact"] < 2 << 20 and ws["deterministic"] > B * E * K * I * 4 and ws["atomic"] > B * E * K * I * 2
+    Y = hk.expert_gather_forward_call(g["X"], g["Wg"], g["Ind"], torch.float32)
+    outs, dXs = {}, {}
+    for mode in ("deterministic", "compact"):
+        with hk.scatter_mode_scope(mode), _abi.launch_log() as log:
+            outs[mode] = hk.expert_scatter_forward_call(Y, g["Ws"], g["Ind"], T, torch.float32)
+            dXs[mode] = hk.expert_gather_backward_call(g["X"], g["Wg"], g["Ind"], Y, torch.float32)[0]
+            again = hk.expert_scatter_forward_call(Y, g["Ws"], g["Ind"], T, torch.float32)
+        assert torch.equal(outs[mode], again)
+        if mode == "compact":
+            assert log.kernels.count("scatter_pass_kernel") == 3 and "segment_sum_kernel" not in log.kernels, log.kernels
+        else:
+            assert "scatter_pass_kernel" not in log.kernels, log.kernels
+    # Zipf: one token takes about a quarter of a batch element's picks; both modes round a token's fp32 sum once
+    counts = torch.bincount(inp["Ind"][0].reshape(-1), minlength=T)
+    assert counts.max() > 0.15 * cfg.E * cfg.K
+    b = 3
+    Indn = inp["Ind"].numpy()
+    ref = O.scatter_forward(np64(Y[b:b + 1]), np64(inp["Ws"]), Indn[b:b + 1], T, acc=np.float64)
+    assert_close(outs["compact"][b:b + 1], ref, cfg.dtype, "C4 out, compact mode")
+    ref = O.gather_backward(np64(inp["X"][b:b + 1]), np64(inp["Wg"]), Indn[b:b + 1], np64(Y[b:b + 1]))[0]
+    assert_close(dXs["compact"][b:b + 1], ref, cfg.dtype, "C4 dX, compact mode")
+    assert_close(dXs["deterministic"][b:b + 1], ref, cfg.dtype, "C4 dX, deterministic mode")
 
 
 def test_scatter_cut_into_uneven_batch_groups():

@@ -90,6 +90,15 @@ SMALL_SHAPES = [
     (8, 64, 64, 64, 32, 32),      # 4096 picks: four passes of 16 experts
 ]
 
+# sizes beyond the one-kernel scatters above that the compact mode's one-kernel scatter in passes takes (16-bit types,
+# reduction 32 / 64 / 128, T <= 1024): 32-pick units, the sums of up to 1024 tokens in registers
+PASS_SHAPES = [
+    (8, 700, 20, 100, 320, 64),   # 2000 picks, ragged units (K = 100), three passes, T > 512
+    (3, 1000, 33, 150, 1024, 32), # 4950 picks, reduction 32, 32 slices
+    (10, 1024, 40, 128, 256, 128),# 5120 picks, reduction 128, T at the limit, five passes of whole experts
+    (2, 600, 7, 300, 128, 128),   # few workgroups (8), one expert spans ten units: a wavefront's units change expert mid-pass
+]
+
 
 @pytest.fixture(params=[False, True], ids=["fastpaths", "generic"])
 def force_generic(request):
@@ -147,6 +156,25 @@ def test_ind_is_never_written():
     assert torch.equal(Ind, keep)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("shape", PASS_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_compact_mode_matches_oracle(shape, dtype):
+    from expertscattergather_amd import _abi
+    B, T, E, K, I, J = shape
+    case = make_case(300 + sum(shape), *shape, dtype)
+    with _abi.launch_log() as log:
+        got = run_all(case, T, mode="compact")
+    assert log.kernels.count("scatter_pass_kernel") == 2, log.kernels          # the scatter forward, and dX
+    ref = oracle_all(case, T)
+    for name in ("Y", "out", "dX", "dWg", "dY", "dWs"):
+        assert_close(got[name], ref[name], dtype, f"compact {name} {shape} {dtype}")
+    d = _abi.Dims(*shape)
+    dt = hk.dtype_to_type_id(dtype)
+    lib = _abi.lib()
+    assert lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, _abi.SCATTER_COMPACT, d, dt) < \
+        lib.egs_workspace_bytes(_abi.OP_GEMM_SCATTER, _abi.SCATTER_DETERMINISTIC, d, dt) // 8
+
+
 def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
     # all picks of every expert land on 3 tokens: long same-token chains
     B, T, E, K, I, J = 4, 64, 8, 48, 96, 40
@@ -168,6 +196,61 @@ def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
     hk.set_scatter_mode("deterministic")
     assert_close(atomic, np64(first), torch.float32, "atomic vs deterministic")
     del junk
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+def test_pass_scatter_with_long_segments_is_ordered(dtype):
+    """The one-kernel scatter in passes (compact mode) under skew: a quarter of a batch element's picks on one token (its
+    segment is dealt to all wavefronts in chunks), a few tokens with 65 .. 500 picks (summed by a wavefront each, in every
+    pass), many with 5 .. 64 (which finish in their threads' own loops), rejected picks, tokens nobody picks; both weight
+    layouts; bitwise repeatable; the kernel is the one asserted."""
+    from expertscattergather_amd import _abi
+    B, T, E, K, I, J = 8, 900, 50, 120, 320, 64
+    case = make_case(23, B, T, E, K, I, J, dtype)
+    g = torch.Generator().manual_seed(4)
+    p = torch.arange(1, T + 1, dtype=torch.float64).pow(-1.2)
+    Ind = torch.multinomial(p.expand(B * E, T), K, replacement=True, generator=g).reshape(B, E, K)
+    Ind = torch.randperm(T, generator=g)[Ind]
+    Ind[Ind == 17] = 18                                     # a token nobody picks
+    Ind[0, 0, 0] = -1; Ind[B - 1, E - 1, K - 1] = T; Ind[3, 7, 50] = 30000
+    counts = torch.bincount(Ind[1][(Ind[1] >= 0) & (Ind[1] < T)].reshape(-1), minlength=T)
+    assert counts.max() > 0.2 * E * K and ((counts > 64) & (counts < 400)).sum() >= 3 and ((counts > 4) & (counts <= 64)).sum() > 20
+    bad = (Ind < 0) | (Ind >= T)
+    safe = Ind.clone(); safe[bad] = 0
+    mask = (~bad).numpy()[..., None]
+    Y, Ws, Wg, Indg = dev(case["Y"]), dev(case["Ws"]), dev(case["Wg"]), dev(Ind)
+    with hk.scatter_mode_scope("compact"):
+        with _abi.launch_log() as log:
+            out = hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32)
+        assert "scatter_pass_kernel" in log.kernels, log.kernels
+        for _ in range(3):
+            assert torch.equal(out, hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32))
+        assert_close(out, O.scatter_forward(np64(case["Y"]) * mask, np64(case["Ws"]), safe.numpy(), T), dtype, "pass scatter, skewed")
+        assert out[:, 17].abs().max().item() == 0.0
+        with _abi.launch_log() as log:
+            dX, _ = hk.expert_gather_backward_call(dev(case["X"]), Wg, Indg, Y, torch.float32)
+        assert "scatter_pass_kernel" in log.kernels, log.kernels
+        assert torch.equal(dX, hk.expert_gather_backward_call(dev(case["X"]), Wg, Indg, Y, torch.float32)[0])
+        assert_close(dX, O.gather_backward(np64(case["X"]), np64(case["Wg"]), safe.numpy(), np64(case["Y"]) * mask)[0], dtype,
+                     "pass scatter as dX, skewed")
+
+
+def test_pass_scatter_with_more_long_tokens_than_slots():
+    """Seventy tokens of a batch element with more than 64 picks each: the first 16 in token order are summed by
+    wavefronts, the others by their threads; repeatable and within tolerance all the same."""
+    B, T, E, K, I, J = 10, 600, 64, 100, 256, 32
+    dtype = torch.bfloat16
+    case = make_case(29, B, T, E, K, I, J, dtype)
+    g = torch.Generator().manual_seed(6)
+    hot = torch.randperm(T, generator=g)[:70]
+    Ind = hot[torch.randint(0, 70, (B, E, K), generator=g)]          # 6400 picks on 70 tokens: ~91 each
+    counts = torch.bincount(Ind[0].reshape(-1), minlength=T)
+    assert (counts > 64).sum() > 64
+    Y, Ws, Indg = dev(case["Y"]), dev(case["Ws"]), dev(Ind)
+    with hk.scatter_mode_scope("compact"):
+        out = hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32)
+        assert torch.equal(out, hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32))
+    assert_close(out, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), Ind.numpy(), T), dtype, "pass scatter, 70 long tokens")
 
 
 def test_multi_pass_scatter_is_bitwise_reproducible_with_hot_tokens():
