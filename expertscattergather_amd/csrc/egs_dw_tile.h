@@ -155,21 +155,24 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
 
     // 16-bit fragment addresses inside a piece ([32 picks][64 or YB bytes]): the lane points at pick 8 g + 4 h + a / 4 and
     // the four columns 4 (a % 4) of a 16-column group, and receives column a of picks 8 g + 4 h .. + 3
-    // The 32-byte units of a row (one 16-column group each) are XOR-swizzled by the pick number so that the four picks
-    // a transpose read touches per 16 lanes fall on different banks: unit ^ (pick / 2 % 2) in the 64-byte rows, unit ^
-    // (pick % 4) in the 128-byte rows.  pick = 8 g + 4 h + a / 4 below, so the key depends on a / 4 only (and on h for
-    // the 64-byte rows, where at1 = at0 + 4 rows keeps pick / 2 % 2).
+    // The 32-byte units of a row (one 16-column group each) are XOR-swizzled by the pick number so that the 16 rows a
+    // transpose read touches (four picks per 16 lanes, lane groups eight picks apart) spread over the banks: eight picks
+    // are 512 or 1024 bytes, a multiple of the banks' 256-byte period, so without a term in pick / 8 the four lane groups
+    // would read the same banks (measured: 52 % of the LDS-active cycles were bank conflicts).  Key of pick p:
+    // (p / 2 % 2) ^ (p / 8 % 2) in the 64-byte rows, (p % 4) ^ (p / 8 % 4) in the 128-byte rows: the 512 bytes of a
+    // read then fall two deep on every bank, the least possible.  p = 8 g + 4 h + a / 4 below.
     // fp32 fragments are single elements: matrix-instruction step k of a 32-pick step takes pick 4 k + g from lane group g,
     // column a of a 16-column group; rows are padded instead of swizzled (dw_tile_xstride).
     const int fr = a >> 2;                              // pick of the lane inside its group of four
-    const int xkey = (fr >> 1) & 1, ykey = YB == 64 ? (fr >> 1) & 1 : fr & 3;
+    const int xkey = ((fr >> 1) & 1) ^ (g & 1), ykey = YB == 64 ? ((fr >> 1) & 1) ^ (g & 1) : (fr & 3) ^ g;
     const int at0 = ES == 2 ? (g * 8 + fr) * 64 + (a & 3) * 8 : g * XS + a * 4, at1 = at0 + 4 * 64;
     const int yat0 = ES == 2 ? (g * 8 + fr) * YB + (a & 3) * 8 : g * YS + a * 4, yat1 = yat0 + 4 * YB;
     // writers: lane holds chunk c (16 bytes; 16-bit: half a unit) of pick p
     const int xp = lane / XL, xcn = lane % XL;
-    const int wr = ES == 2 ? xp * 64 + (((xcn >> 1) ^ ((xp >> 1) & 1)) << 5) + (xcn & 1) * 16 : xp * XS + xcn * 16;
+    const int wr = ES == 2 ? xp * 64 + (((xcn >> 1) ^ ((xp >> 1) & 1) ^ ((xp >> 3) & 1)) << 5) + (xcn & 1) * 16 : xp * XS + xcn * 16;
     const int yp = lane / YL, ycn = lane % YL;
-    const int ywr = ES == 2 ? yp * YB + (((ycn >> 1) ^ (YB == 64 ? (yp >> 1) & 1 : yp & 3)) << 5) + (ycn & 1) * 16
+    // (a load of the 128-byte rows covers eight picks: pick / 8 is the load's number h, added in stage_write)
+    const int ywr = ES == 2 ? yp * YB + (((ycn >> 1) ^ (YB == 64 ? ((yp >> 1) & 1) ^ ((yp >> 3) & 1) : yp & 3)) << 5) + (ycn & 1) * 16
                             : yp * YS + ycn * 16;
     // A step goes registers -> LDS tile (stage_write), LDS tile -> fragments (stage_read), fragments -> MFMAs.  The
     // loop is software-pipelined: the fragments of step s are requested first, then the registers of step s+1 are
@@ -180,7 +183,8 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
 #pragma unroll
         for (int h = 0; h < XN; ++h) *reinterpret_cast<u32x4 *>(st + h * (64 / XL) * XS + wr) = rx[s][h];
 #pragma unroll
-        for (int h = 0; h < YN; ++h) *reinterpret_cast<u32x4 *>(st + XT + h * (64 / YL) * YS + ywr) = ry[s][h];
+        for (int h = 0; h < YN; ++h)
+            *reinterpret_cast<u32x4 *>(st + XT + h * (64 / YL) * YS + (ES == 2 && YB == 128 ? ywr ^ ((h & 3) << 5) : ywr)) = ry[s][h];
     };
     // fragments of a step: 16-bit, one 16-byte operand per 16-column group (8 picks per lane group);
     // fp32, eight single elements per group (one per matrix-instruction step)
