@@ -37,27 +37,37 @@ PROFILES = os.path.join(ROOT, "profiles")
 
 
 def kernel_list(kernels):
-    """'a + b + a + b' -> '2 x (a + b)'; a call that works through batch groups launches the same kernels once per group"""
-    n = len(kernels)
-    for period in range(1, n // 2 + 1):
-        if n % period == 0 and kernels == kernels[:period] * (n // period):
-            return f"{n // period} x ({' + '.join(kernels[:period])})"
-    return " + ".join(kernels)
+    """'a + b + a + b + c' -> '2 x (a + b) + c'; a call that works through batch groups launches the same kernels once per group"""
+    out, i, n = [], 0, len(kernels)
+    while i < n:
+        best = (1, 1)                       # (period, repeats) of the longest repeated run that starts at i
+        for period in range(1, (n - i) // 2 + 1):
+            reps = 1
+            while kernels[i + reps * period:i + (reps + 1) * period] == kernels[i:i + period]:
+                reps += 1
+            if reps > 1 and reps * period > best[0] * best[1]:
+                best = (period, reps)
+        period, reps = best
+        unit = " + ".join(kernels[i:i + period])
+        out.append(f"{reps} x ({unit})" if reps > 1 else unit)
+        i += period * reps
+    return " + ".join(out)
 
 
 def recorded_traffic():
     """HBM-side bytes per launch from the rocprofv3 --pmc summaries under profiles/ (FETCH_SIZE + WRITE_SIZE of
     `bench.py --pmc-probe` runs, each scaled by what the same counter reads for a 64 MiB copy).  Counters cannot be read
     from inside this process, so the figures are the recorded ones: lines
-    `traffic <workload> <launch> <bytes> [<kernel>+<kernel>...]`; the optional last field names the kernels the launch ran
-    when the counters were read, and a figure whose kernels are no longer the ones selected is not reported."""
+    `traffic <workload> <launch> <bytes> <kernel>+<kernel>...`; the last field names the kernels the launch ran when the
+    counters were read (a launch has one line per set of kernels it can select, e.g. per scatter mode), and a figure is
+    reported only for the set of kernels selected now."""
     import glob
     import re
     found = {}
     for path in sorted(glob.glob(os.path.join(PROFILES, "*.md")) + glob.glob(os.path.join(PROFILES, "*.txt"))):
-        for m in re.finditer(r"^\s*traffic (\S+) (\S+) (\d+)(?:[ \t]+(\S+))?\s*$", open(path).read(), flags=re.M):
-            found[(m.group(1), m.group(2))] = {"bytes": int(m.group(3)), "source": os.path.relpath(path, ROOT),
-                                               "kernels": m.group(4).split("+") if m.group(4) else None}
+        for m in re.finditer(r"^\s*traffic (\S+) (\S+) (\d+)[ \t]+(\S+)\s*$", open(path).read(), flags=re.M):
+            found[(m.group(1), m.group(2), tuple(sorted(set(m.group(4).split("+")))))] = {
+                "bytes": int(m.group(3)), "source": os.path.relpath(path, ROOT)}
     return found
 
 
@@ -338,10 +348,10 @@ class Workload:
         # dense matrix peak of the arithmetic type"
         _, nbytes, nflops = self.launch_fns()[lname]
         t_hbm, t_mfma = nbytes / (HBM_PEAK_GBPS * 1e9), nflops / (self.mfma_peak * 1e12)
-        tr = None if self.fp8_act else traffic.get((self.name, lname))
         kernels = self.kernels[lname]
-        if tr is not None and tr["kernels"] is not None and sorted(set(tr["kernels"])) != sorted(set(kernels)):
-            tr = None           # counters were read for other kernels than the ones selected now
+        # counters read for other kernels than the ones selected now say nothing about this launch
+        # (nor do counters read in the ordered modes about the "atomic" mode, whose kernels carry the same names)
+        tr = None if self.fp8_act or self.mode == "atomic" else traffic.get((self.name, lname, tuple(sorted(set(kernels)))))
         common = {"launch": lname, "kernel": kernel_list(kernels), "avg_launch_us": round(t * 1e6, 3),
                   "avg_launch_us_cold": None if t_cold is None else round(t_cold * 1e6, 3),
                   "algorithmic_bytes": nbytes, "algorithmic_flops": nflops,

@@ -271,13 +271,16 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
     __syncthreads();                                    // every wavefront is done with its tables and staging tiles
 
     // lane (a, g) holds dW rows i0 + 16 x + a, columns j0 + 16 y + 4 g .. + 3
-    float *red = reinterpret_cast<float *>(smem);       // [NW][32 i][TJ j]
-    static_assert(32 * TJ * 4 <= kLdsPerWave, "reduction buffer fits");
+    // A row of the exchange buffer is TJ + 4 floats: with rows of 128 or 256 bytes the 16 lanes of a 16-byte write
+    // (16 rows, same columns) would all fall on the same 4 banks, and the column-wise reads of the [E,J,I] layout on one.
+    constexpr int RS = TJ + 4;
+    float *red = reinterpret_cast<float *>(smem);       // [NW][32 i][RS]
+    static_assert(32 * RS * 4 <= kLdsPerWave, "reduction buffer fits");
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
         for (int y = 0; y < NY; ++y)
-            *reinterpret_cast<f32x4 *>(red + wave * (32 * TJ) + (x * 16 + a) * TJ + y * 16 + g * 4) = acc[x][y];
+            *reinterpret_cast<f32x4 *>(red + wave * (32 * RS) + (x * 16 + a) * RS + y * 16 + g * 4) = acc[x][y];
     __syncthreads();
 
     // wavefront tiles are added in wavefront order; 4 consecutive elements of the requested layout per thread
@@ -288,18 +291,18 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
         const int minor4 = (eji ? item & 7 : item % (TJ / 4)) * 4;
         f32x4 v;
         if (!eji) {
-            v = *reinterpret_cast<const f32x4 *>(red + major * TJ + minor4);
+            v = *reinterpret_cast<const f32x4 *>(red + major * RS + minor4);
 #pragma unroll
             for (int w = 1; w < NW; ++w) {
-                const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * (32 * TJ) + major * TJ + minor4);
+                const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * (32 * RS) + major * RS + minor4);
                 v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
             }
         } else {
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                float s1 = red[(minor4 + x) * TJ + major];
+                float s1 = red[(minor4 + x) * RS + major];
 #pragma unroll
-                for (int w = 1; w < NW; ++w) s1 += red[w * (32 * TJ) + (minor4 + x) * TJ + major];
+                for (int w = 1; w < NW; ++w) s1 += red[w * (32 * RS) + (minor4 + x) * RS + major];
                 v[x] = s1;
             }
         }
