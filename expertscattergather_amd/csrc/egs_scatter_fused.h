@@ -76,7 +76,9 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     // slices of one batch element sit on one XCD (ids congruent modulo 8 share an XCD), so that its
     // rows are fetched from memory once
     const int grp = block & 7, idx = block >> 3;
-    const int b = (idx / p.slices) * 8 + grp, slice = idx % p.slices;
+    const int qb = idx / p.slices, slice = idx % p.slices;
+    // XCD grp takes the batch elements 2 grp, 2 grp + 1 of every 16 (a last incomplete block: grp of every 8)
+    const int b = (qb | 1) < ((p.B + 7) >> 3) ? (qb >> 1) * 16 + grp * 2 + (qb & 1) : qb * 8 + grp;
     if (b >= p.B) return;
     const int c0 = slice * kFusedCols;
     const int T = p.T, E = p.E, K = p.K, N = p.N, NP = E * K;
