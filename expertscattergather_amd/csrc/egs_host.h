@@ -103,11 +103,10 @@ int rows_gemm_gather(RowsGemmParams &p, int act_dtype, bool fp8_w, bool w_trans,
 int rows_gemm_scatter(RowsGemmParams &p, int act_dtype, bool w_trans, int epi, hipStream_t s);
 
 // ---- egs_pass_launch.hip: the one-kernel GEMM-scatter in passes (thousands of picks per batch element, 16-bit types)
-struct PassPlan { bool ok; int units_per_pass; size_t lds; int32_t perm_at, seg_at, long_at; };
+struct PassPlan { bool ok; int units_per_pass; size_t lds; };
 PassPlan scatter_pass_plan(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype);
-// `seg` [B][T+1], `perm` [B][E*K]: the routing table of all batch elements, in memory
-int scatter_pass(const void *Y, const void *W, void *Out, const egs_dims *d, int act_dtype, int w_layout, const int32_t *seg,
-                 const int32_t *perm, hipStream_t s);
+int scatter_pass(const void *Y, const void *W, const void *Ind, void *Out, const egs_dims *d, int act_dtype, int ind_dtype,
+                 int w_layout, hipStream_t s);
 
 // ---- egs_dw_launch.hip: tiled weight gradient (general and direct-to-LDS kernels) with its second pass
 int dw_general(const void *Xs, const void *Ys, const void *Ind, void *dW, void *workspace, const egs_dims *d,

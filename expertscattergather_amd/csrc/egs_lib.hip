@@ -120,7 +120,7 @@ struct ScatterPlan {
 //   long-segment records and partial rows, and the product rows in pick order - fp32 in deterministic mode
 //   (fp32 accumulation with one final rounding), the element type in atomic ("fast") mode with 16-bit types
 //   (half the traffic, one extra rounding per pick; the summation order is still fixed).
-//   the one-kernel scatter in passes (SCATTER_PASS) needs the routing table only;
+//   the one-kernel scatter in passes (SCATTER_PASS) needs nothing either (it sorts each pass's picks in LDS);
 enum ScatterPath { SCATTER_FUSED, SCATTER_PASS, SCATTER_ROWS };
 
 ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype, ScatterPath path)
@@ -129,14 +129,13 @@ ScatterPlan plan_scatter(const egs_dims *d, int mode, int act_dtype, ScatterPath
     memset(&pl, 0, sizeof(pl));
     const size_t N = (size_t)d->E * d->K;
     if (mode == EGS_SCATTER_ATOMIC && act_dtype == EGS_F32) return pl;
-    if (path == SCATTER_FUSED) return pl;
+    if (path == SCATTER_FUSED || path == SCATTER_PASS) return pl;
     const size_t row_es = (mode != EGS_SCATTER_ATOMIC || act_dtype == EGS_F32) ? 4 : (size_t)elem_size(act_dtype);
     size_t at = 0;
     pl.seg_off_at = at; at += align_up((size_t)d->B * ((size_t)d->T + 1) * 4, 256);
     pl.perm_at = at;    at += align_up((size_t)d->B * N * 4, 256);
     pl.rank_at = at;    at += align_up((size_t)d->B * N * 4, 256);
     pl.cnt_at = at;     at += d->T > kCsrLdsTokens ? align_up((size_t)d->B * d->T * 4, 256) : 0;
-    if (path == SCATTER_PASS) { pl.bytes = at; return pl; }
     // long segments (tokens picked more than kLongSegment times): records and fp32 partial rows
     pl.long_tab_at = at;  at += align_up((size_t)d->B * long_tab_stride((int)N) * 4, 256);
     pl.long_part_at = at; at += align_up((size_t)d->B * long_max_slots((int)N) * d->I * 4, 256);
@@ -773,9 +772,9 @@ bool scatter_fused_takes(const void *Y, const void *W, const void *Out, const eg
 
 // The one-kernel scatters come first where they apply (they are the fastest there and need no workspace).  Beyond them
 // the product rows go through the workspace, unless the caller asks for the compact mode: the one-kernel scatter in
-// passes keeps them in LDS for up to 32768 picks per batch element, at C4's sizes in 133 us against 106 us (plus the
-// routing table's launch either way) - its token sums, table look-ups and the moves of its operands into matrix-
-// instruction order all go through the one LDS pipe of the compute unit - but with 1 MB of workspace instead of 270 MB.
+// passes keeps them in LDS and sorts each pass's picks there too, for any number of picks per batch element and with no
+// workspace at all - at B16 T1024 E64 K128 I512 J128 in 136 us under Zipf routing and 133 us under even routing, where
+// the product rows through 270 MB of workspace take 120 and 105 us.
 ScatterPath scatter_choose(const void *Y, const void *W, const void *Out, const egs_dims *d, int act_dtype, int mode)
 {
     if (scatter_fused_takes(Y, W, Out, d, act_dtype)) return SCATTER_FUSED;
@@ -967,6 +966,8 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     }
 
     if (fused) return scatter_fused(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, dw, dwt, s, use);   // small experts: one kernel
+    // compact mode, thousands of picks per batch element: one kernel in passes, nothing in the workspace
+    if (path == SCATTER_PASS) return scatter_pass(Y, W, Ind, Out, d, act_dtype, ind_dtype, w_layout, s);
 
     // routing table (picks in token order) + product rows in pick order, then one fixed-order
     // gather-and-sum per token that writes every output row exactly once
@@ -976,12 +977,6 @@ int gemm_scatter_impl(const void *Y, const void *W, const void *Ind, void *Out, 
     int32_t *cnt = d->T > kCsrLdsTokens ? (int32_t *)(ws + pl.cnt_at) : nullptr;
     int32_t *long_tab = (int32_t *)(ws + pl.long_tab_at);
     float *long_part = (float *)(ws + pl.long_part_at);
-    if (path == SCATTER_PASS) {
-        // compact mode, thousands of picks per batch element: the table as a launch of its own, then one kernel
-        const int rc_tab = launch_routing_table(Ind, ind_dtype, d, seg_off, perm, rank_tmp, cnt, nullptr, s);
-        if (rc_tab != EGS_OK) return rc_tab;
-        return scatter_pass(Y, W, Out, d, act_dtype, w_layout, seg_off, perm, s);
-    }
     void *rows = ws + pl.rows_at;
     bool rows_f32 = (mode != EGS_SCATTER_ATOMIC);
     // small experts: the sort rides along with the product when its histograms are small

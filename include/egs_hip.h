@@ -78,13 +78,14 @@ typedef enum egs_w_layout {
 typedef enum egs_scatter_mode {
     EGS_SCATTER_DETERMINISTIC = 0,  /* fixed summation order, bitwise reproducible, no atomics   */
     EGS_SCATTER_ATOMIC = 1,         /* fp32 atomic accumulation, order of additions unspecified  */
-    EGS_SCATTER_COMPACT = 2         /* DETERMINISTIC with the smallest workspace: where the sizes allow (16-bit types, reduction
-                                     * 32 / 64 / 128, T <= 1024, up to 32768 picks per batch element) the product rows stay on
-                                     * the compute unit and the workspace holds the routing table only - the reference's
-                                     * kernel (egs/triton_kernels.py:156-247) has no intermediate either, and its README
-                                     * (README.md:36) sells the path on memory; at large shapes slower than DETERMINISTIC,
-                                     * which spends B*E*K*I*4 bytes of workspace on fp32 product rows; same tolerances, its
-                                     * own (fixed) order of additions */
+    EGS_SCATTER_COMPACT = 2         /* DETERMINISTIC without a workspace: where the sizes allow (16-bit types, reduction
+                                     * 32 / 64 / 128, output columns a multiple of 32, T <= 1024, more than 1024 picks per
+                                     * batch element) the product rows stay on the compute unit, the picks are sorted there
+                                     * too, and egs_workspace_bytes returns 0 - the reference's kernel
+                                     * (egs/triton_kernels.py:156-247) has no intermediate either, and its README
+                                     * (README.md:36) sells the path on memory; DETERMINISTIC spends B*E*K*I*4 bytes of
+                                     * workspace on fp32 product rows and is faster at large shapes with even routing;
+                                     * same tolerances, its own (fixed) order of additions */
 } egs_scatter_mode;
 
 typedef enum egs_op {

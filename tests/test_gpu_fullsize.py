@@ -118,14 +118,14 @@ def test_c3_long_sequence_bf16():
 def test_c4_zipf_routing_both_modes():
     check_large("C4", ["deterministic", "atomic"])
     # compact mode: the configuration's scatters (forward, and dX in the gather's backward) run in one kernel each, product
-    # rows in LDS and a workspace of the routing table only; the other modes go through product rows in the workspace
+    # rows and sorted picks in LDS and no workspace at all; the other modes go through product rows in the workspace
     from expertscattergather_amd import _abi
     cfg, inp, g = gpu_inputs("C4")
     B, T, E, K, I, J = cfg.dims
     d = _abi.Dims(*cfg.dims)
     ws = {m: _abi.lib().egs_workspace_bytes(_abi.OP_GEMM_SCATTER, v, d, _abi.BF16) for m, v in
           (("deterministic", 0), ("atomic", 1), ("compact", 2))}
-    assert ws["compact"] < 2 << 20 and ws["deterministic"] > B * E * K * I * 4 and ws["atomic"] > B * E * K * I * 2
+    assert ws["compact"] == 0 and ws["deterministic"] > B * E * K * I * 4 and ws["atomic"] > B * E * K * I * 2
     Y = hk.expert_gather_forward_call(g["X"], g["Wg"], g["Ind"], torch.float32)
     outs, dXs = {}, {}
     for mode in ("deterministic", "compact"):

@@ -201,9 +201,8 @@ def test_deterministic_mode_is_bitwise_reproducible_with_hot_tokens():
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
 def test_pass_scatter_with_long_segments_is_ordered(dtype):
     """The one-kernel scatter in passes (compact mode) under skew: a quarter of a batch element's picks on one token (its
-    segment is dealt to all wavefronts in chunks), a few tokens with 65 .. 500 picks (summed by a wavefront each, in every
-    pass), many with 5 .. 64 (which finish in their threads' own loops), rejected picks, tokens nobody picks; both weight
-    layouts; bitwise repeatable; the kernel is the one asserted."""
+    16-token block's list holds a quarter of every pass), a few tokens with 65 .. 500 picks, many with 5 .. 64, rejected
+    picks, tokens nobody picks; both weight layouts; bitwise repeatable; the kernel is the one asserted."""
     from expertscattergather_amd import _abi
     B, T, E, K, I, J = 8, 900, 50, 120, 320, 64
     case = make_case(23, B, T, E, K, I, J, dtype)
@@ -236,8 +235,8 @@ def test_pass_scatter_with_long_segments_is_ordered(dtype):
 
 
 def test_pass_scatter_with_more_long_tokens_than_slots():
-    """Seventy tokens of a batch element with more than 64 picks each: the first 16 in token order are summed by
-    wavefronts, the others by their threads; repeatable and within tolerance all the same."""
+    """Seventy tokens of a batch element with more than 64 picks each, spread over the token blocks of all wavefronts:
+    repeatable and within tolerance."""
     B, T, E, K, I, J = 10, 600, 64, 100, 256, 32
     dtype = torch.bfloat16
     case = make_case(29, B, T, E, K, I, J, dtype)
@@ -251,6 +250,57 @@ def test_pass_scatter_with_more_long_tokens_than_slots():
         out = hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32)
         assert torch.equal(out, hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32))
     assert_close(out, O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), Ind.numpy(), T), dtype, "pass scatter, 70 long tokens")
+
+
+def test_pass_scatter_keeps_a_value_that_is_not_finite_to_its_token():
+    """Compact mode adds with matrix instructions whose selector is 0 or 1; 0 x inf would be NaN for the other tokens of a
+    16-token block, so a pass with a product that is not finite takes its sums without multiplications: the value reaches
+    the token that picked it and nobody else, and every other row is what it is without that pick."""
+    from expertscattergather_amd import _abi
+    B, T, E, K, I, J = 8, 600, 20, 100, 64, 64           # T > 512: beyond the one-kernel scatter of small experts
+    dtype = torch.bfloat16
+    case = make_case(41, B, T, E, K, I, J, dtype)
+    Ind = case["Ind"].clone()
+    Yc = case["Y"].clone()
+    b, e, k = 2, 7, 33
+    t_bad = int(Ind[b, e, k])
+    Yc[b, e, k, :] = float("inf")
+    Yc[b + 1, e, k, 3] = float("nan")
+    t_nan = int(Ind[b + 1, e, k])
+    Y, Ws, Indg = dev(Yc), dev(case["Ws"]), dev(Ind)
+    with hk.scatter_mode_scope("compact"), _abi.launch_log() as log:
+        out = hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32)
+        again = hk.expert_scatter_forward_call(Y, Ws, Indg, T, torch.float32)
+    assert log.kernels.count("scatter_pass_kernel") == 2, log.kernels
+    finite = torch.isfinite(out.float())
+    assert not finite[b, t_bad].any() and not finite[b + 1, t_nan].any()       # inf . W has both signs in every column: inf or nan
+    finite[b, t_bad] = True; finite[b + 1, t_nan] = True
+    assert finite.all(), "a value that is not finite leaked to another token"
+    assert torch.equal(torch.nan_to_num(out.float(), 0.0, 0.0, 0.0), torch.nan_to_num(again.float(), 0.0, 0.0, 0.0))
+    Yz = Yc.clone(); Yz[b, e, k, :] = 0; Yz[b + 1, e, k, :] = 0
+    ref = O.scatter_forward(np64(Yz), np64(case["Ws"]), Ind.numpy(), T)
+    got = out.clone(); got[b, t_bad] = 0; got[b + 1, t_nan] = 0
+    ref[b, t_bad] = 0; ref[b + 1, t_nan] = 0
+    assert_close(got, ref, dtype, "pass scatter beside a value that is not finite")
+
+
+@pytest.mark.parametrize("ind_dtype", [torch.int32, torch.int16], ids=["int32", "int16"])
+def test_pass_scatter_reads_narrow_indices(ind_dtype):
+    """The compact mode sorts each pass's picks from Ind itself (no routing table in memory): every index width, ragged
+    K (units of 32 picks with a short last one), T not a multiple of 16."""
+    from expertscattergather_amd import _abi
+    B, T, E, K, I, J = 9, 777, 37, 45, 96, 32
+    dtype = torch.float16
+    case = make_case(43, B, T, E, K, I, J, dtype)
+    Ind = case["Ind"].clone()
+    Ind[0, 0, 0] = -1; Ind[4, 5, 6] = T
+    bad = (Ind < 0) | (Ind >= T)
+    safe = Ind.clone(); safe[bad] = 0
+    mask = (~bad).numpy()[..., None]
+    with hk.scatter_mode_scope("compact"), _abi.launch_log() as log:
+        out = hk.expert_scatter_forward_call(dev(case["Y"]), dev(case["Ws"]), dev(Ind.to(ind_dtype)), T, torch.float32)
+    assert "scatter_pass_kernel" in log.kernels, log.kernels
+    assert_close(out, O.scatter_forward(np64(case["Y"]) * mask, np64(case["Ws"]), safe.numpy(), T), dtype, f"pass scatter, {ind_dtype}")
 
 
 def test_multi_pass_scatter_is_bitwise_reproducible_with_hot_tokens():
