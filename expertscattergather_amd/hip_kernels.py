@@ -72,9 +72,10 @@ def _check_mode(mode: str) -> str:
 
 def set_scatter_mode(mode: str) -> None:
     """Process-wide default: 'deterministic' (fixed summation order, bitwise reproducible), 'atomic' (fp32
-    atomics; 16-bit types: product rows kept in the element type) or 'compact' (deterministic with the smallest
-    scratch: where the sizes allow, product rows never leave the compute unit and the scratch is the routing table
-    only - 1 MB instead of 270 MB at B16 T1024 E64 K128 I512 J128 - at large shapes slower).  A module's ``scatter_mode`` attribute and
+    atomics; 16-bit types: product rows kept in the element type) or 'compact' (deterministic without
+    scratch memory: where the sizes allow, product rows never leave the compute unit and the picks are sorted there
+    too - 0 bytes instead of 270 MB at B16 T1024 E64 K128 I512 J128 - slower per launch at large shapes with even
+    routing).  A module's ``scatter_mode`` attribute and
     ``scatter_mode_scope`` take precedence.  A forward call binds the mode in force to its autograd node: the
     backward of that call runs in the same mode whatever is set by then."""
     global _scatter_mode
