@@ -177,6 +177,36 @@ def test_bench_refuses_more_than_one_gpu():
     assert "one GPU" in res.stderr and res.stdout.strip() == ""
 
 
+def test_bench_names_repeated_kernel_groups_and_reads_recorded_traffic_by_kernels():
+    """bench.py reports, per launch, the kernels the library's launch log named; a call that works through batch groups
+    repeats a group of kernels, which the name collapses.  The HBM-side traffic of a launch is a recorded figure
+    (rocprofv3 cannot run inside the benchmark): a line per (workload, launch, set of kernels) under profiles/, used only
+    when the kernels are the ones selected now."""
+    import importlib.util
+    import os
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("egs_bench", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    assert bench.kernel_list(["a"]) == "a" and bench.kernel_list([]) == ""
+    assert bench.kernel_list(["a", "b", "a", "b"]) == "2 x (a + b)"
+    assert bench.kernel_list(["a", "b"] * 8 + ["c"]) == "8 x (a + b) + c"
+    assert bench.kernel_list(["t", "a", "b", "a", "b", "c", "c"]) == "t + 2 x (a + b) + 2 x (c)"
+    found = bench.recorded_traffic()
+    assert ("C2", "expert_gather_backward", ("scatter_fused_dwtile_table_kernel",)) in found
+    # one launch, two sets of kernels (deterministic and compact mode), two figures
+    c4 = {k[2]: v["bytes"] for k, v in found.items() if k[:2] == ("C4", "expert_scatter_forward")}
+    assert c4[("scatter_pass_kernel",)] < c4[("rows_gemm_dl_kernel", "segment_sum_kernel")] // 4
+    # every recorded line names its kernels, and its source file is where the line is
+    for path in sorted(os.listdir(os.path.join(root, "profiles"))):
+        text = open(os.path.join(root, "profiles", path)).read()
+        for line in re.findall(r"^\s*traffic .*$", text, flags=re.M):
+            assert re.match(r"^\s*traffic C[1-5] expert_\w+ \d+ [\w+]+\s*$", line), (path, line)
+    for key, rec in found.items():
+        assert os.path.exists(os.path.join(root, rec["source"])), key
+
+
 def test_compute_dtype_follows_the_reference_kernels():
     # out_type float16 / bfloat16: both operands are cast to it (reference egs/triton_kernels.py:122-127);
     # float32: operands stay as they are - a shared 16-bit type is multiplied in that type, mixed types meet in float32
