@@ -27,7 +27,7 @@ from . import _abi
 __all__ = [
     "create_kernels", "dtype_to_type_id", "ExpertGatherFunction", "ExpertScatterFunction",
     "set_scatter_mode", "get_scatter_mode", "scatter_mode_scope", "expert_gather_fp8w_forward", "expert_gather_fp8_forward", "validate_indices",
-    "register_reference_namespace", "release_workspaces", "expert_mlp_forward",
+    "register_reference_namespace", "release_workspaces", "expert_mlp_forward", "expert_mlp", "ExpertMLPFunction",
     "set_routing_table_cache", "invalidate_routing_table",
 ]
 
@@ -747,6 +747,14 @@ _TORCH_ACT = {
     _abi.ACT_GELU_TANH: lambda y: torch.nn.functional.gelu(y, approximate="tanh"),
 }
 
+# derivative of the activation applied to an incoming gradient: (grad, input) -> grad * act'(input), torch's own kernels
+_TORCH_ACT_BACKWARD = {
+    _abi.ACT_RELU: lambda g, y: torch.ops.aten.threshold_backward(g, y, 0),
+    _abi.ACT_GELU: lambda g, y: torch.ops.aten.gelu_backward(g, y, approximate="none"),
+    _abi.ACT_SILU: lambda g, y: torch.ops.aten.silu_backward(g, y),
+    _abi.ACT_GELU_TANH: lambda g, y: torch.ops.aten.gelu_backward(g, y, approximate="tanh"),
+}
+
 
 def _mlp_block_pays(B: int, E: int, K: int, I: int, J: int, act: int) -> bool:
     """Measured on MI355X (bf16): the one kernel wins while its workgroups fit one round of the device (256) and the
@@ -812,6 +820,52 @@ def _mlp_forward_impl(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.
     with torch.no_grad():
         Y = _TORCH_ACT[act](_gather_forward_impl(X, W_gather, Ind, torch.float32))
         return _scatter_forward_impl(Y, W_scatter, Ind, T, torch.float32)
+
+
+class ExpertMLPFunction(torch.autograd.Function):
+    """Trainable ``scatter(act(gather(X, W_gather, Ind)), W_scatter, Ind, T)`` that keeps no ``Y[B,E,K,J]`` between
+    forward and backward (the layer pattern of the reference, test_speed.ipynb:73-75, as one autograd node).
+
+    Forward: `expert_mlp_forward` (one kernel for small experts, the rows between the two products never in memory).
+    Saved for backward: ``X``, the two weights and ``Ind`` only - none of the ``B*E*K*J`` activations the two separate
+    Functions save (``Y`` for the activation, ``act(Y)`` for the scatter).  Backward recomputes the gather product
+    (one more launch) and then runs what the separate Functions would: the scatter's backward on ``act(Y)``, the
+    activation's derivative (torch), the gather's backward.  The recomputed rows are rounded to the element type before
+    the activation (the one-kernel forward rounds after it), so for activations other than relu/none the ``act(Y)`` the weight
+    gradient sees can differ from the forward's in the last bit."""
+
+    @staticmethod
+    def forward(ctx, X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor, activation="relu"):
+        create_kernels()
+        if activation not in _ACTIVATIONS:
+            raise ValueError(f"activation must be one of {sorted(k for k in _ACTIVATIONS if k)}, got {activation!r}")
+        ctx.save_for_backward(X, W_gather, W_scatter, Ind)
+        ctx.act = _ACTIVATIONS[activation]
+        ctx.scatter_mode = _mode_to_bind()
+        return expert_mlp_forward(X, W_gather, W_scatter, Ind, activation)
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, grad_out: torch.Tensor):
+        X, Wg, Ws, Ind = ctx.saved_tensors
+        Y = expert_gather_forward_call(X, Wg, Ind, torch.float32)
+        A = Y.relu_() if ctx.act == _abi.ACT_RELU else _TORCH_ACT[ctx.act](Y)    # relu's derivative can be read off its result
+        grad_Y, grad_Ws = expert_scatter_backward_call(A, Ws, Ind, grad_out, torch.float32)
+        del A
+        if ctx.act != _abi.ACT_NONE:
+            grad_Y = _TORCH_ACT_BACKWARD[ctx.act](grad_Y, Y)
+        del Y
+        if ctx.scatter_mode is None:
+            grad_X, grad_Wg = expert_gather_backward_call(X, Wg, Ind, grad_Y, torch.float32)
+        else:
+            with scatter_mode_scope(ctx.scatter_mode):
+                grad_X, grad_Wg = expert_gather_backward_call(X, Wg, Ind, grad_Y, torch.float32)
+        return grad_X, grad_Wg, grad_Ws, None, None
+
+
+def expert_mlp(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor, activation="relu") -> torch.Tensor:
+    """Differentiable block, see `ExpertMLPFunction`.  X [B,T,I], W_gather [E,I,J], W_scatter [E,J,I], Ind [B,E,K] -> [B,T,I]."""
+    return ExpertMLPFunction.apply(X, W_gather, W_scatter, Ind, activation)
 
 
 def validate_indices(Ind: torch.Tensor, T: int) -> int:

@@ -838,6 +838,40 @@ def test_inference_block_composes_what_the_kernel_does_not_take():
         hk.expert_mlp_forward(X, Wg, Ws, Ind, "softmax")
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("act", ["relu", "silu", "none"])
+@pytest.mark.parametrize("shape,dtype", [((8, 96, 16, 24, 128, 64), torch.bfloat16),     # the one-kernel forward
+                                         ((3, 40, 6, 9, 64, 96), torch.float16),          # J = 96: composed forward
+                                         ((2, 33, 5, 7, 24, 40), torch.float32)],
+                         ids=["block-bf16", "composed-f16", "composed-f32"])
+def test_trainable_block_keeps_no_rows_and_matches_the_chain_rule(shape, dtype, act):
+    """hip_kernels.expert_mlp: output and the three gradients against the oracle's chain with every stored stage
+    rounded to the element type (the activation and its derivative from torch in float64 on the CPU), and nothing of
+    size B*E*K*J saved for backward."""
+    B, T, E, K, I, J = shape
+    case = make_case(47, B, T, E, K, I, J, dtype)
+    X, Wg, Ws = (dev(case[k]).requires_grad_(True) for k in ("X", "Wg", "Ws"))
+    Ind = dev(case["Ind"])
+    out = hk.expert_mlp(X, Wg, Ws, Ind, act)
+    assert {t.data_ptr() for t in out.grad_fn.saved_tensors} <= {t.data_ptr() for t in (X, Wg, Ws, Ind)}
+    out.backward(dev(case["dOut"]))
+
+    rnd = lambda v: torch.from_numpy(np.asarray(v)).to(dtype).to(torch.float64).numpy()
+    Xn, Wgn, Wsn, dOn = (np64(case[k]) for k in ("X", "Wg", "Ws", "dOut")); Indn = case["Ind"].numpy()
+    fn = {"none": lambda v: v, "relu": torch.relu, "silu": torch.nn.functional.silu}[act]
+    Yo = torch.from_numpy(rnd(O.gather_forward(Xn, Wgn, Indn))).requires_grad_(True)
+    Ao = fn(Yo)
+    An = rnd(Ao.detach().numpy())
+    one_kernel = dtype is not torch.float32 and J in (32, 64)
+    assert_close(out, _mlp_oracle(case, T, act, dtype, stored_y=not one_kernel), dtype, "trainable block, out")
+    dAo, dWso = O.scatter_backward(An, Wsn, Indn, dOn)
+    assert_close(Ws.grad, dWso, dtype, "trainable block, dWs")
+    dYo = rnd(torch.autograd.grad(Ao, Yo, torch.from_numpy(rnd(dAo)))[0].numpy()) if act != "none" else rnd(dAo)
+    dXo, dWgo = O.gather_backward(Xn, Wgn, Indn, dYo)
+    assert_close(X.grad, dXo, dtype, "trainable block, dX")
+    assert_close(Wg.grad, dWgo, dtype, "trainable block, dWg")
+
+
 def test_inference_block_is_a_traceable_op():
     hk.create_kernels()
     B, T, E, K, I, J = 8, 48, 8, 16, 64, 32
