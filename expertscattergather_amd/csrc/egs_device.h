@@ -391,4 +391,17 @@ __device__ __forceinline__ bool decode_tile_expert(int bid, int tiles_per_expert
     return tile < tiles_per_expert;
 }
 
+// The three maps behind one switch.  `rows_share`: 0 = experts map to XCDs (decode_expert_tile); 1 = row tiles map to
+// XCDs in groups of eight (decode_tile_expert); 2 or 4 = there are 8 / rows_share row tiles per expert in all, each
+// owns rows_share XCDs, and the experts are dealt among those (few row tiles must not leave XCDs without work).
+__device__ __forceinline__ bool decode_rows_block(int bid, int rows_share, int tiles_per_expert, int E, int &e, int &tile)
+{
+    if (rows_share == 0) return decode_expert_tile(bid, tiles_per_expert, E, e, tile);
+    if (rows_share == 1) return decode_tile_expert(bid, tiles_per_expert, E, e, tile);
+    const int xcd = bid & 7, slot = bid >> 3;
+    tile = xcd / rows_share;
+    e = slot * rows_share + xcd % rows_share;
+    return e < E && tile < tiles_per_expert;
+}
+
 }  // namespace egs

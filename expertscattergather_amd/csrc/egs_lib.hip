@@ -241,6 +241,26 @@ struct DwTileJob {
 // element in a stable order by token.  Built once per Ind by a gather forward, read by the one-kernel scatters that follow.
 struct RoutingTable { int32_t *seg, *perm; };
 
+
+// Workgroup -> (expert, row tile) map of the small-expert row kernels (decode_rows_block): which operand is worth keeping
+// XCD-local - the source rows, each read by ~E*K/T experts and fetched from beyond the L2 once per XCD that uses them,
+// or W(e), fetched once per XCD that runs one of the expert's row tiles.  Row tiles take the XCDs only where that leaves none
+// idle: in groups of eight, or 2 / 4 of them on 4 / 2 XCDs each.
+int rows_xcd_map(const egs_dims *d, int R, int N, int es, int tiles_per_e)
+{
+    const double picks_per_token = (double)d->E * d->K / (d->T > 0 ? d->T : 1);
+    const double x_bytes = (double)d->B * d->T * R * es, w_bytes = (double)d->E * R * N * es;
+    const double by_expert = x_bytes * (picks_per_token < 8 ? (picks_per_token < 1 ? 1 : picks_per_token) : 8) + w_bytes;
+    const double by_rows = x_bytes + w_bytes * (tiles_per_e < 8 ? tiles_per_e : 8);
+    if (by_rows >= by_expert) return 0;
+    if (tiles_per_e == 2 || tiles_per_e == 4) return 8 / tiles_per_e;
+    return (tiles_per_e % 8 == 0 || tiles_per_e > 16) ? 1 : 0;
+}
+int rows_xcd_blocks(int map, int tiles_per_e, int E)
+{
+    return map == 0 ? 8 * ceil_div(E, 8) * tiles_per_e : map == 1 ? 8 * ceil_div(tiles_per_e, 8) * E : 8 * ceil_div(E, map);
+}
+
 bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, const egs_dims *d, int64_t ldx_b,
                        int64_t ldx_t, int act_dtype, int w_dtype, int ind_dtype, int w_layout, SmallRowsJob &j,
                        const RoutingTable *build = nullptr)
@@ -260,13 +280,7 @@ bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, c
     p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
     p.tiles_per_e = (int)((Me + 255) / 256);
     if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return false;
-    {   // which operand is worth keeping XCD-local: the source rows (each read by ~E*K/T experts) or W[e]
-        const double picks_per_token = (double)d->E * d->K / d->T;
-        const double x_bytes = (double)d->B * d->T * R * 2, w_bytes = (double)d->E * R * N * 2;
-        const double by_expert = x_bytes * (picks_per_token < 8 ? (picks_per_token < 1 ? 1 : picks_per_token) : 8) + w_bytes;
-        const double by_rows = x_bytes + w_bytes * (p.tiles_per_e < 8 ? p.tiles_per_e : 8);
-        p.rows_share_xcd = by_rows < by_expert;
-    }
+    p.rows_share_xcd = rows_xcd_map(d, R, N, 2, p.tiles_per_e);
     j.R = R; j.act_dtype = act_dtype; j.gather = true; j.out_f32 = false; j.lds = 0;
     j.nmajor = (w_layout == EGS_W_EIJ);                 // [E,I,J] = [E,R,N]
     if (build != nullptr) {             // the routing table of a later scatter rides along: B more workgroups, first in line
@@ -274,7 +288,7 @@ bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, c
         p.seg_off = build->seg; p.perm = build->perm;
         j.lds = csr_count_lds(d->T, 4);
     }
-    j.blocks = (p.rows_share_xcd ? 8 * ceil_div(p.tiles_per_e, 8) * p.E : 8 * ceil_div(p.E, 8) * p.tiles_per_e) + p.csr_blocks;
+    j.blocks = rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E) + p.csr_blocks;
     return true;
 }
 
@@ -460,9 +474,9 @@ int gather_small_f32(const void *X, const void *W, const void *Ind, void *Y, con
     p.lda_b = ldx_b; p.lda_t = ldx_t; p.ind_dtype = ind_dtype;
     p.tiles_per_e = (int)((Me + 255) / 256);
     if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return EGS_OK;
-    p.rows_share_xcd = 0;               // W(e) is fetched once per workgroup: experts share an XCD
+    p.rows_share_xcd = rows_xcd_map(d, R, N, 4, p.tiles_per_e);
     if (build != nullptr) { p.csr_blocks = d->B; p.seg_off = build->seg; p.perm = build->perm; }
-    const int blocks = 8 * ceil_div(p.E, 8) * p.tiles_per_e + p.csr_blocks;
+    const int blocks = rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E) + p.csr_blocks;
     used = true;
     const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]
     switch (R) {
@@ -1408,8 +1422,10 @@ int egs_expert_scatter_backward(const void *Y, const void *W, const void *Ind, c
         SmallRowsJob g8 = gj;
         const int64_t Me = (int64_t)d->B * d->K;
         g8.p.tiles_per_e = (int)((Me + 511) / 512);
-        if (g8.p.tiles_per_e % 8 != 0) g8.p.rows_share_xcd = 0;     // row tiles map to XCDs in groups of 8 only
-        g8.blocks = g8.p.rows_share_xcd ? 8 * ceil_div(g8.p.tiles_per_e, 8) * g8.p.E : 8 * ceil_div(g8.p.E, 8) * g8.p.tiles_per_e;
+        // (row tiles on the XCDs in groups of eight only: with four row tiles on two XCDs each this launch measured
+        // 11.4 against 11.05 us at B64 T256 E32 K32 I128 J64 - its other half reads the same rows expert by expert)
+        g8.p.rows_share_xcd = g8.p.tiles_per_e % 8 == 0 ? rows_xcd_map(d, d->I, d->J, 2, g8.p.tiles_per_e) : 0;
+        g8.blocks = rows_xcd_blocks(g8.p.rows_share_xcd, g8.p.tiles_per_e, g8.p.E);
         if ((int64_t)g8.blocks + dwt.blocks <= INT32_MAX / 2) return launch_rows_small_job(g8, nullptr, &dwt, s);
     }
     const bool dw_tile = w_elems > 0 && make_dw_tile(grad_Out, Y, Ind, grad_W, d, ldg_b, ldg_t, dtype, dtype, ind_dtype, EGS_W_EJI, dwt,

@@ -38,7 +38,7 @@ struct SmallRowsParams {
     int64_t lda_b, lda_t;
     int32_t ind_dtype;
     int32_t tiles_per_e;    // workgroups (256 picks each) per expert
-    int32_t rows_share_xcd; // 1: row tiles map to XCDs (source rows reused across experts), 0: experts map to XCDs
+    int32_t rows_share_xcd; // workgroup -> (expert, row tile) map, see decode_rows_block: 0 experts map to XCDs, 1 / 2 / 4 row tiles do (source rows reused across experts)
     // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
     int32_t csr_blocks;
     int32_t *seg_off, *perm, *rank_tmp, *long_tab;
@@ -61,8 +61,7 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     }
     int e, tile;
     const int bid = block - p.csr_blocks;
-    if (p.rows_share_xcd ? !decode_tile_expert(bid, p.tiles_per_e, p.E, e, tile)
-                         : !decode_expert_tile(bid, p.tiles_per_e, p.E, e, tile)) return;
+    if (!decode_rows_block(bid, p.rows_share_xcd, p.tiles_per_e, p.E, e, tile)) return;       // uniform per workgroup
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: scalar address work
     const int a = lane & 15, g = lane >> 4;
     const int Me = p.B * p.K;
