@@ -818,6 +818,7 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     if (use != nullptr && fused_reads_table(fp, d, act_dtype)) { p.tab_seg = use->seg; p.tab_perm = use->perm; }
     p.perm_at = (int32_t)((int64_t)fp.experts_per_pass * d->K * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
+    p.zero_at = (int32_t)scatter_fused_zero_at(d->T, (int)NP, fp.experts_per_pass * d->K);
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
     if (act_dtype == EGS_F32)
         return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, nullptr, s)

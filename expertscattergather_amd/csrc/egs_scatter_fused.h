@@ -45,6 +45,7 @@ struct ScatterFusedParams {
     int32_t ind_dtype;
     int32_t slices;         // N / kFusedCols
     int32_t perm_at, cnt_at;    // byte offsets of the table and of the sort's counters in dynamic LDS (rows start at 0)
+    int32_t zero_at;            // ... and of 128 bytes of zeros (128-byte aligned), scatter_fused_zero_at()
     int32_t experts_per_pass;   // MULTI: experts whose product rows are in LDS at a time (E otherwise)
     // TABLE: routing table built beforehand (seg [B][T+1], perm [B][E*K]); the workgroup copies its batch element's part
     // into LDS instead of sorting the picks itself
@@ -55,10 +56,15 @@ constexpr int kFusedMaxPasses = 4;
 constexpr int kFusedMultiTokens = 8;    // MULTI: tokens per thread (64 threads groups of 8 walk the tokens) -> T <= 512
 
 // LDS bytes: product rows (of `rows` picks at a time), table of all NP picks, counters of the sort (one histogram
-// per wavefront + offsets)
+// per wavefront + offsets), a row of zeros
+__host__ __device__ inline size_t scatter_fused_zero_at(int T, int NP, int rows)
+{
+    const size_t at = (size_t)rows * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)(kFusedThreads / 64 + 1) * T + 1) * 4 + 64;
+    return (at + 127) & ~(size_t)127;
+}
 __host__ __device__ inline size_t scatter_fused_lds(int T, int NP, int rows)
 {
-    return (size_t)rows * kFusedCols * 4 + (size_t)NP * 4 + ((size_t)(kFusedThreads / 64 + 1) * T + 1) * 4 + 64;
+    return scatter_fused_zero_at(T, NP, rows) + kFusedCols * 4;
 }
 __host__ __device__ inline size_t scatter_fused_lds(int T, int NP) { return scatter_fused_lds(T, NP, NP); }
 
@@ -68,7 +74,14 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     // KS = reduction length in MFMA steps of four 16-byte chunks: 32 elements of a 16-bit type, 16 of fp32
     constexpr int ES = TT::ES, VEC = TT::VEC;
     constexpr int R = 4 * VEC * KS;
-    constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 32-pick) units in flight per wavefront
+    constexpr int kFusedDepth = KS == 4 ? 2 : 4;         // (expert, 32-pick) units a wavefront has registers for
+    // Units requested ahead of the one being multiplied.  One pass: a single one - the wavefronts of a CU then take turns
+    // at its one address path, which is what bounds this phase (about 200 cycles of it per unit with the 4-byte pieces of an
+    // [E,R,N] weight; with all four units requested up front a wavefront spent 5000 cycles issuing before it multiplied
+    // anything, 8.3 against 9.8 us at B64 T256 E32 K32 I128 J64 together with the summing loop below).  In passes: all.
+    constexpr int kAhead = MULTI ? kFusedDepth : 1;
+    // a table that this workgroup parks itself (TABLE, one pass) is parked as row addresses, see (2)
+    constexpr bool kEncoded = TABLE && !MULTI;
     // the wavefront index is made known as uniform: units, experts and base addresses derived from it are then
     // scalar work, and the loads take a scalar base with a per-lane 32-bit offset
     const int tid = (int)threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -88,6 +101,7 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     int32_t *cnt = reinterpret_cast<int32_t *>(smem + p.cnt_at);
     constexpr int NWV = kFusedThreads / 64;
     const int32_t *seg = cnt + NWV * T;                 // token offsets left there by the sort
+    if (!MULTI && tid < kFusedCols) reinterpret_cast<float *>(smem + p.zero_at)[tid] = 0.f;     // read after the barrier before (2)
 
     // ---------------- (1) units of work of this wavefront: (expert, pair of 16-pick row tiles); the weight
     // fragments of a unit serve both row tiles
@@ -202,20 +216,23 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
 #pragma unroll
         for (int x = 0; x < SV; ++x) sv[x] = gseg[min(tid + x * kFusedThreads, T)];
 #pragma unroll
-        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
+        for (int d = 0; d < kAhead; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
         int32_t *seg_w = cnt + NWV * T;
         // entries are clamped to what a table of these sizes can hold: whatever a caller hands over (a table of other
         // indices, memory that was never filled), every loop below ends and every access stays inside the workgroup's rows
 #pragma unroll
         for (int x = 0; x < PV; ++x)
-            if (tid + x * kFusedThreads < NP) perm[tid + x * kFusedThreads] = min(max(pv[x], 0), NP - 1);
+            if (tid + x * kFusedThreads < NP) {
+                const int q = min(max(pv[x], 0), NP - 1);
+                perm[tid + x * kFusedThreads] = kEncoded ? (q << 7) | ((q & 7) << 4) : q;
+            }
 #pragma unroll
         for (int x = 0; x < SV; ++x)
             if (tid + x * kFusedThreads <= T) seg_w[tid + x * kFusedThreads] = min(max(sv[x], 0), NP);
     } else {
     csr_count_body(cnt, b, 0, tid, kFusedThreads, p.Ind, p.ind_dtype, T, NP, nullptr, perm, nullptr, nullptr, [&]() {
 #pragma unroll
-        for (int d = 0; d < kFusedDepth; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
+        for (int d = 0; d < kAhead; ++d) load_unit(buf[d], wave + NWV * d, 0, min(EP, E));
     });
     }
 
@@ -236,28 +253,51 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
         for (int u0 = wave; u0 < E * KT2; u0 += NWV * kFusedDepth) {
 #pragma unroll
             for (int d = 0; d < kFusedDepth; ++d) {
+                // the request for the unit kAhead further on goes out before this one is multiplied: a CU's wavefronts
+                // then take turns at its one address path instead of all queueing there first and multiplying afterwards
+                if constexpr (kAhead < kFusedDepth) load_unit(buf[(d + kAhead) % kFusedDepth], u0 + NWV * (d + kAhead), 0, E);
                 compute_unit(buf[d], u0 + NWV * d, E);
-                load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth, 0, E);
+                if constexpr (kAhead == kFusedDepth) load_unit(buf[d], u0 + NWV * d + NWV * kFusedDepth, 0, E);
             }
         }
         __syncthreads();
 
-        // ---------------- (2) per token: add its product rows in table order; 8 threads x 4 columns per token
-        for (int t = tid >> 3; t < T; t += kFusedThreads >> 3) {
+        // ---------------- (2) per token: add its product rows in table order; 4 threads x 8 columns per token.
+        // The table entries of a segment are read four at a time without looking at its end (what follows in LDS is the next
+        // segment or the sort's counters: inside the allocation either way); an entry past the end selects a row of zeros
+        // instead of its own, so that the additions need no condition.  Entry q stands for byte (q << 7) | ((q & 7) << 4),
+        // chunk 0 of row q in the rows' XOR order: a thread's two chunks are one XOR away each.  (The phase is bound by
+        // vector-ALU issue - two wavefronts per SIMD, all in it at once - so it is written for few instructions per pick.)
+        const uint32_t c2 = (uint32_t)(tid & 3) << 5, zero_sel = (uint32_t)p.zero_at;
+        for (int t = tid >> 2; t < T; t += kFusedThreads >> 2) {
             const int s0 = seg[t], s1 = seg[t + 1];
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
             for (int s = s0; s < s1; s += 4) {
-                int q[4];
-                f32x4 v[4];
+                const int n = s1 - s;
+                uint32_t en[4];
+                f32x4 v[4][2];
 #pragma unroll
-                for (int x = 0; x < 4; ++x) q[x] = perm[min(s + x, s1 - 1)];
+                for (int x = 0; x < 4; ++x) en[x] = (uint32_t)perm[s + x];
 #pragma unroll
-                for (int x = 0; x < 4; ++x) v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)q[x] * kFusedCols)[cc ^ (q[x] & 7)];
+                for (int x = 0; x < 4; ++x) {
+                    const uint32_t at = kEncoded ? en[x] : (en[x] << 7) | ((en[x] & 7u) << 4);
+                    const uint32_t sel = (x < n) ? at : zero_sel;
+                    v[x][0] = *reinterpret_cast<const f32x4 *>(smem + (sel ^ c2));
+                    v[x][1] = *reinterpret_cast<const f32x4 *>(smem + (sel ^ (c2 | 16u)));
+                }
 #pragma unroll
-                for (int x = 0; x < 4; ++x)
-                    if (s + x < s1) sum += v[x];
+                for (int x = 0; x < 4; ++x) { lo += v[x][0]; hi += v[x][1]; }
             }
-            store_row(t, sum);
+            char *dst = p.out + (((size_t)b * T + t) * N + c0 + (tid & 3) * 8) * ES;
+            if constexpr (ES == 4) {
+                reinterpret_cast<f32x4 *>(dst)[0] = lo;
+                reinterpret_cast<f32x4 *>(dst)[1] = hi;
+            } else {
+                u32x4 w;
+                w[0] = pack2<TT>(lo[0], lo[1]); w[1] = pack2<TT>(lo[2], lo[3]);
+                w[2] = pack2<TT>(hi[0], hi[1]); w[3] = pack2<TT>(hi[2], hi[3]);
+                *reinterpret_cast<u32x4 *>(dst) = w;
+            }
         }
     } else {
         // ---------------- (1) + (2) in passes over groups of EP experts.  A thread keeps, for each of its tokens, the
