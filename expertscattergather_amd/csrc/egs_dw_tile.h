@@ -14,9 +14,9 @@
 // the opposite of what the matrix instruction wants (per lane: 8 consecutive picks of one column).  Per
 // 32-pick step a wavefront fetches the 64-byte pieces of 32 gathered Xs rows and the 64- or 128-byte pieces of
 // 32 Ys rows with 16-byte buffer loads (adjacent lanes take adjacent chunks of a pick's piece: one access per
-// row), keeps a whole chunk of picks in flight in registers, drops each step into a wavefront-private LDS tile
-// as [pick][column] and reads the fragments back with the LDS transpose read.  No barrier in the main loop.  Row byte offsets come from a table in LDS that the wavefront decodes
-// from Ind one chunk ahead; picks that do not exist (bad index, ragged end) get an offset outside the buffer
+// row), one step ahead of the step it multiplies, drops each step into a wavefront-private LDS tile
+// as [pick][column] and reads the fragments back with the LDS transpose read.  No barrier in the main loop.  Row byte
+// offsets come from a table in LDS that the wavefront decodes from Ind one chunk (128 or 256 picks) ahead; picks that do not exist (bad index, ragged end) get an offset outside the buffer
 // descriptor and arrive as zeros on both sides.
 //
 // Replaces the reference's expert_gather_scatter_dW_kernel (egs/triton_kernels.py:261-356), which reduces
@@ -41,7 +41,7 @@ struct DwTileParams {
 };
 
 // `ES` = bytes per element (2, or 4 for fp32, whose pieces are twice as long and whose fragments are read untransposed)
-// picks whose rows a wavefront keeps in flight at a time (registers: 16 or 24 per 32-pick step; 32 or 48 in fp32)
+// picks whose row offsets a wavefront decodes at a time (a chunk; its steps have registers of their own: 16 or 24 per 32-pick step; 32 or 48 in fp32)
 __host__ __device__ constexpr int dw_tile_chunk(int TJ, int ES = 2) { return (TJ == 32 ? 256 : 128) / (ES / 2); }
 // byte strides of a pick's piece inside a staging tile.  16-bit: dense (the transpose reads are XOR-swizzled instead).
 // fp32: 48 or 80 floats, so that the four picks a 4-byte fragment read touches (16 lanes each) fall on different banks
@@ -217,37 +217,47 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
     };
     auto chunk_len = [&](int c) { return c < nchunks ? min(CH, w_end - w_begin - c * CH) : 0; };
 
+    // Steps whose rows are requested ahead of the step being multiplied: one.  Not the whole chunk: a CU's wavefronts
+    // share one address path, a wavefront cannot drop its first step into LDS before its own requests are accepted, and
+    // with a chunk (8 or 4 steps) requested up front all of them queued there first (B64 T256 E32 K32 I128 J64, the launches
+    // that carry this body: 11.1 -> 10.5 us and 17.1 -> 16.1 us; two steps ahead the same, three and four slower).
+    constexpr int P = 1;
+    static_assert(P <= NS, "a chunk has at least one step");
+    auto issue_step = [&](int c, int sp) {              // step sp >= 0 counted from the start of chunk c; may lie in the next chunks
+        const int cc = c + sp / NS, ss = sp % NS;
+        if (ss * 32 < chunk_len(cc)) issue(cc, ss);
+    };
     if (nchunks > 0) {
         load_idx(0);
         store_tab(0);
         if (nchunks > 1) { load_idx(1); }
-        const int len0 = chunk_len(0);
 #pragma unroll
-        for (int s = 0; s < NS; ++s)
-            if (s * 32 < len0) issue(0, s);
+        for (int s = 0; s < P; ++s) issue_step(0, s);
         if (nchunks > 1) { store_tab(1); }
         if (nchunks > 2) load_idx(2);
         stage_write(0);
-        if (nchunks > 1) issue(1, 0);
+        issue_step(0, P);
     }
     for (int c = 0; c < nchunks; ++c) {
-        const int len = chunk_len(c), len1 = chunk_len(c + 1), len2 = chunk_len(c + 2);
-        // the table of chunk c+2 replaces that of chunk c, whose loads have all been issued; its index words were
-        // requested a chunk ago
-        if (len2 > 0) store_tab(c + 2);
-        if (c + 3 < nchunks) load_idx(c + 3);
+        const int len = chunk_len(c), len1 = chunk_len(c + 1);
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
+            // the table of chunk c+2 replaces that of chunk c once the last step of chunk c has been requested (at the
+            // step before this one); its index words were requested a chunk ago
+            if (s == NS - P) {
+                if (chunk_len(c + 2) > 0) store_tab(c + 2);
+                if (c + 3 < nchunks) load_idx(c + 3);
+            }
             if (s * 32 < len) {
                 Frag pf[2], qf[NY];
                 stage_read(s, pf, qf);
                 __builtin_amdgcn_sched_barrier(0);
                 if (s + 1 < NS && (s + 1) * 32 < len) {
                     stage_write(s + 1);
-                    if ((s + 1) * 32 < len1) issue(c + 1, s + 1);
+                    issue_step(c, s + 1 + P);
                 } else if (len1 > 0) {                  // last step of the chunk: the next chunk's first step
                     stage_write(0);
-                    if (len2 > 0) issue(c + 2, 0);
+                    issue_step(c + 1, P);
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (ES == 2) {
