@@ -292,40 +292,41 @@ __device__ __forceinline__ void dw_tile_body(const DwTileParams &p, const int bl
         for (int y = 0; y < NY; ++y)
             *reinterpret_cast<f32x4 *>(red + wave * (32 * RS) + (x * 16 + a) * RS + y * 16 + g * 4) = acc[x][y];
     __syncthreads();
-
     // wavefront tiles are added in wavefront order; 4 consecutive elements of the requested layout per thread
     const bool eji = p.dw_layout != 0;
     for (int item = tid; item < 8 * TJ; item += NW * 64) {
-        // EIJ: major = i (32 of them), TJ / 4 groups of four j;  EJI: major = j (TJ of them), 8 groups of four i
-        const int major = eji ? item >> 3 : item / (TJ / 4);
-        const int minor4 = (eji ? item & 7 : item % (TJ / 4)) * 4;
-        f32x4 v;
-        if (!eji) {
-            v = *reinterpret_cast<const f32x4 *>(red + major * RS + minor4);
+        // a thread sums four consecutive j of one row i over the wavefronts.  [E,I,J]: consecutive threads take consecutive
+        // groups of j (one 16-byte piece of the output each); [E,J,I]: consecutive threads take consecutive i, whose four
+        // elements go out one by one, each next to its neighbour thread's (rows of the exchange buffer are 4 banks apart:
+        // 16 lanes x 16 bytes cover the banks once)
+        const int gi_l = eji ? item & 31 : item / (TJ / 4);
+        const int gj_l = (eji ? item >> 5 : item % (TJ / 4)) * 4;
+        f32x4 v = *reinterpret_cast<const f32x4 *>(red + gi_l * RS + gj_l);
 #pragma unroll
-            for (int w = 1; w < NW; ++w) {
-                const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * (32 * RS) + major * RS + minor4);
-                v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+        for (int w = 1; w < NW; ++w) {
+            const f32x4 u = *reinterpret_cast<const f32x4 *>(red + w * (32 * RS) + gi_l * RS + gj_l);
+            v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+        }
+        const int gi = i0 + gi_l, gj = j0 + gj_l;
+        if (gi >= p.I || gj >= p.J) continue;           // J % 4 == 0: a group of four j is inside or outside
+        if (!eji) {
+            const size_t at = ((size_t)e * p.I + gi) * p.J + gj;
+            if (p.out_dtype == 0) {
+                *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.dW) + at) = v;
+            } else {
+                u32x2 w2;
+                w2[0] = p.out_dtype == 1 ? pack2<ElemF16>(v[0], v[1]) : pack2<ElemBF16>(v[0], v[1]);
+                w2[1] = p.out_dtype == 1 ? pack2<ElemF16>(v[2], v[3]) : pack2<ElemBF16>(v[2], v[3]);
+                *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.dW) + at) = w2;
             }
         } else {
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                float s1 = red[(minor4 + x) * RS + major];
-#pragma unroll
-                for (int w = 1; w < NW; ++w) s1 += red[w * (32 * RS) + (minor4 + x) * RS + major];
-                v[x] = s1;
+                const size_t at = ((size_t)e * p.J + gj + x) * p.I + gi;
+                if (p.out_dtype == 0) reinterpret_cast<float *>(p.dW)[at] = v[x];
+                else reinterpret_cast<uint16_t *>(p.dW)[at] =
+                         (uint16_t)((p.out_dtype == 1 ? pack2<ElemF16>(v[x], 0.f) : pack2<ElemBF16>(v[x], 0.f)) & 0xffffu);
             }
-        }
-        const int gi = i0 + (eji ? minor4 : major), gj = j0 + (eji ? major : minor4);
-        if (gi >= p.I || gj >= p.J) continue;           // I % 4 == 0 and J % 4 == 0: a group of 4 is inside or outside
-        const size_t at = eji ? ((size_t)e * p.J + gj) * p.I + gi : ((size_t)e * p.I + gi) * p.J + gj;
-        if (p.out_dtype == 0) {
-            *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.dW) + at) = v;
-        } else {
-            u32x2 w2;
-            w2[0] = p.out_dtype == 1 ? pack2<ElemF16>(v[0], v[1]) : pack2<ElemBF16>(v[0], v[1]);
-            w2[1] = p.out_dtype == 1 ? pack2<ElemF16>(v[2], v[3]) : pack2<ElemBF16>(v[2], v[3]);
-            *reinterpret_cast<u32x2 *>(reinterpret_cast<uint16_t *>(p.dW) + at) = w2;
         }
     }
 }
