@@ -44,7 +44,7 @@ struct MlpFusedParams {
     int64_t ldx_b, ldx_t;
     int32_t ind_dtype;
     int32_t slices;         // I / kFusedCols
-    int32_t perm_at, cnt_at;    // as in ScatterFusedParams
+    int32_t perm_at, cnt_at, zero_at;   // as in ScatterFusedParams
     int32_t act;            // MlpAct
 };
 
@@ -70,6 +70,7 @@ __device__ __forceinline__ void mlp_fused_body(const MlpFusedParams &p, const in
     int32_t *cnt = reinterpret_cast<int32_t *>(smem + p.cnt_at);
     constexpr int NWV = kFusedThreads / 64;
     const int32_t *seg = cnt + NWV * T;
+    if (tid < kFusedCols) reinterpret_cast<float *>(smem + p.zero_at)[tid] = 0.f;       // read after the barrier before the sums
 
     const int KT2 = (K + 31) >> 5;
     const int units = E * KT2;                          // (expert, 32 picks); a wavefront takes units wave, wave + 8, ...
@@ -251,26 +252,32 @@ __device__ __forceinline__ void mlp_fused_body(const MlpFusedParams &p, const in
     }
     __syncthreads();
 
-    // ---------------- per token: add its product rows in table order; 8 threads x 4 columns per token
-    const int cc = tid & 7;
-    for (int t = tid >> 3; t < T; t += kFusedThreads >> 3) {
+    // ---------------- per token: add its product rows in table order; 4 threads x 8 columns per token, four table entries
+    // at a time read without looking at the segment's end, those past it replaced by a row of zeros (the loop of
+    // scatter_fused_body, which is bound by vector-ALU issue)
+    const uint32_t c2 = (uint32_t)(tid & 3) << 5, zero_sel = (uint32_t)p.zero_at;
+    for (int t = tid >> 2; t < T; t += kFusedThreads >> 2) {
         const int s0 = seg[t], s1 = seg[t + 1];
-        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
         for (int s = s0; s < s1; s += 4) {
-            int q[4];
-            f32x4 v[4];
+            const int n = s1 - s;
+            uint32_t en[4];
+            f32x4 v[4][2];
 #pragma unroll
-            for (int x = 0; x < 4; ++x) q[x] = perm[min(s + x, s1 - 1)];
+            for (int x = 0; x < 4; ++x) en[x] = (uint32_t)perm[s + x];
 #pragma unroll
-            for (int x = 0; x < 4; ++x) v[x] = reinterpret_cast<const f32x4 *>(rows + (size_t)q[x] * kFusedCols)[cc ^ (q[x] & 7)];
+            for (int x = 0; x < 4; ++x) {
+                const uint32_t sel = (x < n) ? (en[x] << 7) | ((en[x] & 7u) << 4) : zero_sel;
+                v[x][0] = *reinterpret_cast<const f32x4 *>(smem + (sel ^ c2));
+                v[x][1] = *reinterpret_cast<const f32x4 *>(smem + (sel ^ (c2 | 16u)));
+            }
 #pragma unroll
-            for (int x = 0; x < 4; ++x)
-                if (s + x < s1) sum += v[x];
+            for (int x = 0; x < 4; ++x) { lo += v[x][0]; hi += v[x][1]; }
         }
-        u32x2 w;
-        w[0] = pack2<TT>(sum[0], sum[1]);
-        w[1] = pack2<TT>(sum[2], sum[3]);
-        *reinterpret_cast<u32x2 *>(p.out + (((size_t)b * T + t) * N + c0 + cc * 4) * 2) = w;
+        u32x4 w;
+        w[0] = pack2<TT>(lo[0], lo[1]); w[1] = pack2<TT>(lo[2], lo[3]);
+        w[2] = pack2<TT>(hi[0], hi[1]); w[3] = pack2<TT>(hi[2], hi[3]);
+        *reinterpret_cast<u32x4 *>(p.out + (((size_t)b * T + t) * N + c0 + (tid & 3) * 8) * 2) = w;
     }
 }
 

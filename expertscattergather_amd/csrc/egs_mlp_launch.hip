@@ -103,6 +103,7 @@ int egs_expert_mlp_forward(const void *X, const void *Wg, const void *Ws, const 
     p.slices = pl.slices;
     p.perm_at = (int32_t)(NP * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
+    p.zero_at = (int32_t)scatter_fused_zero_at(d->T, (int)NP, (int)NP);
     p.act = activation;
     hipStream_t s = (hipStream_t)stream;
     return dtype == EGS_BF16 ? launch_mlp_tt<ElemBF16>(p, d->I, d->J, pl.lds, (int)pl.blocks, s)

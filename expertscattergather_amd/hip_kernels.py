@@ -757,14 +757,16 @@ _TORCH_ACT_BACKWARD = {
 
 
 def _mlp_block_pays(B: int, E: int, K: int, I: int, J: int, act: int) -> bool:
-    """Measured on MI355X (bf16): the one kernel wins while its workgroups fit one round of the device (256) and the
-    activation is cheap or the (expert, 32-pick) units few - its four slice workgroups per batch element each repeat
-    the activation, and exponentials run at a quarter of the vector rate.  B64 T256 E32 K32 I128 J64, block / separate
-    launches: relu 22.9 / 27.4 us, silu 26.4 / 27.9, gelu 30.4 / 28.4; E16: 14.5 / 24.8, 17.1 / 24.5, 19.3 / 25.0;
+    """Measured on MI355X (bf16, one graph replay per call): the one kernel wins while its workgroups fit one round of the
+    device (256), the batch is large enough (its time hardly depends on the batch: every workgroup walks all E*K picks of
+    its batch element, while the separate launches shrink with it) and the activation is cheap or the (expert, 32-pick)
+    units few - its four slice workgroups per batch element each repeat the activation, and exponentials run at a quarter
+    of the vector rate.  B64 T256 E32 K32 I128 J64, block / separate launches: relu 27.5 / 30.5 us, silu 31.0 / 31.6, gelu
+    33.9 / 31.6; E16: 19.0 / 22.1, 21.4 / 22.2, 23.7 / 22.7; I64 J32: relu 21.3 / 22.9; B32: relu 25.3 / 24.1;
     B128 relu: 43.3 / 41.6 us."""
     blocks = 8 * ((B + 7) // 8) * (I // 32)
     cheap = act in (_abi.ACT_NONE, _abi.ACT_RELU)
-    return blocks <= 256 and (cheap or E * ((K + 31) // 32) <= 16)
+    return blocks <= 256 and B >= 48 and (cheap or E * ((K + 31) // 32) <= 16)
 
 
 def expert_mlp_forward(X: torch.Tensor, W_gather: torch.Tensor, W_scatter: torch.Tensor, Ind: torch.Tensor,
