@@ -246,6 +246,16 @@ struct RoutingTable { int32_t *seg, *perm; };
 // XCD-local - the source rows, each read by ~E*K/T experts and fetched from beyond the L2 once per XCD that uses them,
 // or W(e), fetched once per XCD that runs one of the expert's row tiles.  Row tiles take the XCDs only where that leaves none
 // idle: in groups of eight, or 2 / 4 of them on 4 / 2 XCDs each.
+// whether the routing table that rides in a gather launch is built by two workgroups per batch element
+// (csr_count_half_body) instead of one: its shares must fit the registers and its counters a modest piece of LDS, there must
+// be picks enough to split, and the launch must not grow beyond what the device holds at once (two of these kernels'
+// workgroups fit a CU)
+bool table_split_pays(const egs_dims *d, int nwaves, int gather_blocks, int round_blocks)
+{
+    const int64_t N = (int64_t)d->E * d->K;
+    return N >= 256 && N <= (int64_t)nwaves * 1024 && csr_half_lds(d->T, nwaves) <= 64 * 1024 &&
+           (int64_t)gather_blocks + 2 * (int64_t)d->B <= round_blocks;
+}
 int rows_xcd_map(const egs_dims *d, int R, int N, int es, int tiles_per_e)
 {
     const double picks_per_token = (double)d->E * d->K / (d->T > 0 ? d->T : 1);
@@ -287,6 +297,10 @@ bool make_gather_small(const void *X, const void *W, const void *Ind, void *Y, c
         p.csr_blocks = d->B;
         p.seg_off = build->seg; p.perm = build->perm;
         j.lds = csr_count_lds(d->T, 4);
+        // ... or 2 B, each ranking half of the picks (the ranking is what the build consists of, and the gather's workgroups
+        // alone take less time than one workgroup's whole table: B64 T256 E32 K32, 6.8 -> 6.3 us for the launch)
+        const int gather_blocks = rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E);
+        if (table_split_pays(d, 4, gather_blocks, 512)) { p.csr_blocks = 2 * d->B; p.csr_split = 1; j.lds = csr_half_lds(d->T, 4); }
     }
     j.blocks = rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E) + p.csr_blocks;
     return true;
@@ -433,7 +447,8 @@ int launch_gather_small_f32_ks(const SmallRowsParams &p, int blocks, hipStream_t
     constexpr int TQ = 2, threads = 64 * (16 / TQ);
     static_assert(threads == 64 * kSmallF32Waves, "wavefronts per workgroup");
     size_t lds = rows_small_f32_lds(16 * KS, p.N);
-    if (p.csr_blocks > 0 && csr_count_lds(p.T, kSmallF32Waves) > lds) lds = csr_count_lds(p.T, kSmallF32Waves);
+    const size_t csr_lds = p.csr_split ? csr_half_lds(p.T, kSmallF32Waves) : csr_count_lds(p.T, kSmallF32Waves);
+    if (p.csr_blocks > 0 && csr_lds > lds) lds = csr_lds;
     switch (p.N / 16) {
     case 1: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 1, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
     case 2: hipLaunchKernelGGL((rows_small_f32_kernel<W_NMAJOR, KS, 2, TQ>), dim3(blocks), dim3(threads), lds, s, p); break;
@@ -475,7 +490,10 @@ int gather_small_f32(const void *X, const void *W, const void *Ind, void *Y, con
     p.tiles_per_e = (int)((Me + 255) / 256);
     if ((int64_t)8 * (ceil_div(d->E, 8) + 1) * (p.tiles_per_e + 8) > INT32_MAX / 2) return EGS_OK;
     p.rows_share_xcd = rows_xcd_map(d, R, N, 4, p.tiles_per_e);
-    if (build != nullptr) { p.csr_blocks = d->B; p.seg_off = build->seg; p.perm = build->perm; }
+    if (build != nullptr) {
+        p.csr_blocks = d->B; p.seg_off = build->seg; p.perm = build->perm;
+        if (table_split_pays(d, kSmallF32Waves, rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E), 512)) { p.csr_blocks = 2 * d->B; p.csr_split = 1; }
+    }
     const int blocks = rows_xcd_blocks(p.rows_share_xcd, p.tiles_per_e, p.E) + p.csr_blocks;
     used = true;
     const bool nmajor = (w_layout == EGS_W_EIJ);        // [E,I,J] = [E,R,N]

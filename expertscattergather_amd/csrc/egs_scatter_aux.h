@@ -306,6 +306,140 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
     emit_long_tokens(tok_start, T, N, long_tab, out_b, tid, nthreads);
 }
 
+// The same table built by TWO workgroups per batch element (`h` = 0 or 1), for the case where it rides in a launch that has
+// compute units to spare: the ranking (eight ballot rounds per 64-pick chunk) is what the build consists of, and each
+// workgroup ranks only one half of the picks - the lower pick numbers (h = 0) or the upper ones - and merely counts the other
+// half with LDS atomics (counts do not depend on the order of arrival).  Both compute the same segment offsets; a token's
+// segment lists the lower half's picks before the upper half's, i.e. in increasing pick number as csr_count_body does.
+// Workgroup 0 writes seg_off, each writes its half of perm.  LDS: (2 NW + 1) T + 1 int32 (csr_half_lds).  Requires
+// N <= NW * 1024 (a wavefront's share of a half in registers) - checked by the host.
+__host__ __device__ constexpr size_t csr_half_lds(int T, int nwaves) { return ((size_t)(2 * nwaves + 1) * T + 1) * 4; }
+
+__device__ __forceinline__ void csr_count_half_body(int32_t *sh, int b, int h, int tid, int nthreads, const void *Ind,
+                                                    int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off, int32_t *perm)
+{
+    constexpr int MAXC = 8, MAXO = 8;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = nthreads >> 6;
+    int32_t *hist = sh + (size_t)wave * T;              // own half: this wavefront's counters
+    int32_t *oth = sh + (size_t)(NW + wave) * T;        // other half: this wavefront's counts
+    int32_t *tok_start = sh + (size_t)2 * NW * T;       // [T + 1]
+    int32_t *own_at = sh + (size_t)NW * T;              // after the prefix: where the own half starts inside a token's segment
+    const int split = min(N, ((N + 1) / 2 + 63) & ~63);
+    const int own_begin = h ? split : 0, own_end = h ? N : split;
+    const int oth_begin = h ? 0 : split, oth_end = h ? split : N;
+    const int64_t base_pick = (int64_t)b * N;
+    const int slice = ((own_end - own_begin + NW - 1) / NW + 63) & ~63;
+    const int q_begin = own_begin + wave * slice, q_end = min(own_end, q_begin + slice);
+
+    int32_t tk[MAXC], rk[MAXC];
+    uint64_t tw[MAXC], ow[MAXO];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        tw[c] = 0;
+        if (c * kWave < slice) tw[c] = load_index_word(Ind, ind_dtype, base_pick + min(q_begin + c * kWave + lane, N - 1));
+    }
+#pragma unroll
+    for (int i = 0; i < MAXO; ++i) {
+        ow[i] = 0;
+        if (oth_begin + i * nthreads < oth_end)         // uniform
+            ow[i] = load_index_word(Ind, ind_dtype, base_pick + min(oth_begin + i * nthreads + tid, N - 1));
+    }
+    for (int i = lane; i < T; i += kWave) { cnt_store(&hist[i], 0); cnt_store(&oth[i], 0); }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        const int q = q_begin + c * kWave + lane;
+        int32_t t = -1;
+        if (c * kWave < slice) {
+            const int64_t raw = decode_index_word(tw[c], Ind, ind_dtype, base_pick + min(q, N - 1));
+            t = (raw < 0 || raw >= (int64_t)T) ? -1 : (int32_t)raw;
+        }
+        tk[c] = q < q_end ? t : -1;
+        rk[c] = 0;
+    }
+    const int nbits = T > 1 ? 32 - __clz(T - 1) : 0;
+    const uint64_t lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c) {
+        if (q_begin + c * kWave < q_end) {              // uniform
+            const int32_t t = tk[c];
+            uint64_t same = __ballot(t >= 0);
+            for (int bit = 0; bit < nbits; ++bit) {
+                const bool one = (t >> bit) & 1;
+                const uint64_t bal = __ballot(one);
+                same &= one ? bal : ~bal;
+            }
+            if (t >= 0) {
+                const int rank = __popcll(same & lt_mask), group = __popcll(same);
+                const int start = cnt_load(&hist[t]);
+                rk[c] = start + rank;
+                if (rank == group - 1) cnt_store(&hist[t], start + group);
+            }
+            __builtin_amdgcn_wave_barrier();
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < MAXO; ++i) {
+        const int q = oth_begin + i * nthreads + tid;
+        if (oth_begin + i * nthreads < oth_end) {
+            const int64_t raw = decode_index_word(ow[i], Ind, ind_dtype, base_pick + min(q, N - 1));
+            if (q < oth_end && raw >= 0 && raw < (int64_t)T)
+                __hip_atomic_fetch_add(&oth[(int32_t)raw], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __syncthreads();
+
+    constexpr int kMaxWaves = 16;
+    for (int t = tid; t < T; t += nthreads) {
+        int c[kMaxWaves], o = 0;
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) {
+            c[w] = w < NW ? sh[(size_t)w * T + t] : 0;
+            o += w < NW ? sh[(size_t)(NW + w) * T + t] : 0;
+        }
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) {
+            if (w < NW) sh[(size_t)w * T + t] = run;
+            run += c[w];
+        }
+        tok_start[t] = run + o;
+        own_at[t] = h ? o : 0;
+    }
+    __syncthreads();
+    {   // exclusive scan of the totals over tokens, as in csr_count_body
+        __shared__ int32_t part_total_half[16];
+        const int tw_ = ((T + NW - 1) / NW + 63) & ~63;
+        const int t_begin = wave * tw_, t_end = min(T, t_begin + tw_);
+        int running = 0;
+        for (int t0 = t_begin; t0 < t_end; t0 += kWave) {
+            const int t = t0 + lane;
+            const int c = t < t_end ? tok_start[t] : 0;
+            const int incl = wave_inclusive_scan(c, lane);
+            if (t < t_end) tok_start[t] = running + incl - c;
+            running += __shfl(incl, kWave - 1, kWave);
+        }
+        if (lane == 0) part_total_half[wave] = running;
+        __syncthreads();
+        int before = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < kMaxWaves; ++w) {
+            const int c = w < NW ? part_total_half[w] : 0;
+            if (w < wave) before += c;
+            total += c;
+        }
+        for (int t = t_begin + lane; t < t_end; t += kWave) tok_start[t] += before;
+        if (tid == 0) tok_start[T] = total;
+    }
+    __syncthreads();
+    if (h == 0)
+        for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)b * (T + 1) + t] = tok_start[t];
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c)
+        if (tk[c] >= 0) perm[base_pick + tok_start[tk[c]] + own_at[tk[c]] + hist[tk[c]] + rk[c]] = q_begin + c * kWave + lane;
+}
+
+
 static __global__ __launch_bounds__(1024) void csr_count_kernel(const void *Ind, int32_t ind_dtype, int32_t T, int32_t N,
                                                          int32_t *seg_off, int32_t *perm, int32_t *rank_tmp,
                                                          int32_t *long_tab)

@@ -39,8 +39,9 @@ struct SmallRowsParams {
     int32_t ind_dtype;
     int32_t tiles_per_e;    // workgroups (256 picks each) per expert
     int32_t rows_share_xcd; // workgroup -> (expert, row tile) map, see decode_rows_block: 0 experts map to XCDs, 1 / 2 / 4 row tiles do (source rows reused across experts)
-    // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body
-    int32_t csr_blocks;
+    // routing-table build riding along (csr_blocks = B, or 0): see csr_count_body; csr_split: two workgroups per batch
+    // element (csr_blocks = 2 B), see csr_count_half_body
+    int32_t csr_blocks, csr_split;
     int32_t *seg_off, *perm, *rank_tmp, *long_tab;
 };
 
@@ -55,8 +56,12 @@ __device__ __forceinline__ void rows_small_body(const SmallRowsParams &p, const 
     constexpr int OES = OUT_F32 ? 4 : 2;        // output element size
     static_assert(!(GATHER && OUT_F32), "gather results are stored in the element type");
     if (block < p.csr_blocks) {             // uniform per workgroup; 0 unless a routing table rides along
-        csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
-                       p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
+        if (p.csr_split)
+            csr_count_half_body(sh_cnt_small, block >> 1, block & 1, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
+                                p.E * p.K, p.seg_off, p.perm);
+        else
+            csr_count_body(sh_cnt_small, block, block, (int)threadIdx.x, 64 * WPB, p.Ind, p.ind_dtype, p.T,
+                           p.E * p.K, p.seg_off, p.perm, p.rank_tmp, p.long_tab);
         return;
     }
     int e, tile;

@@ -30,8 +30,12 @@ __global__ __launch_bounds__(64 * (16 / TQ)) void rows_small_f32_kernel(SmallRow
     int bid = (int)blockIdx.x;
     // routing-table build of a later scatter riding along (csr_blocks = B, or 0): one workgroup per batch element, first in line
     if (bid < p.csr_blocks) {
-        csr_count_body(reinterpret_cast<int32_t *>(w_lds), bid, bid, (int)threadIdx.x, NTHREADS, p.Ind, p.ind_dtype, p.T,
-                       p.E * p.K, p.seg_off, p.perm, nullptr, nullptr);
+        if (p.csr_split)
+            csr_count_half_body(reinterpret_cast<int32_t *>(w_lds), bid >> 1, bid & 1, (int)threadIdx.x, NTHREADS, p.Ind,
+                                p.ind_dtype, p.T, p.E * p.K, p.seg_off, p.perm);
+        else
+            csr_count_body(reinterpret_cast<int32_t *>(w_lds), bid, bid, (int)threadIdx.x, NTHREADS, p.Ind, p.ind_dtype, p.T,
+                           p.E * p.K, p.seg_off, p.perm, nullptr, nullptr);
         return;
     }
     bid -= p.csr_blocks;

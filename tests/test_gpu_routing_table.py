@@ -69,12 +69,17 @@ def test_results_do_not_depend_on_the_table(shape, dtype, ind_dtype):
     assert_close(tabled[1], O.scatter_forward(np64(case["Y"]), np64(case["Ws"]), case["Ind"].to(torch.int64).numpy(), T), dtype, "out")
 
 
+@pytest.mark.parametrize("shape", [(5, 50, 9, 11, 64, 32),        # 99 picks: one workgroup per batch element builds the table
+                                   (4, 300, 40, 25, 64, 32),      # 1000 picks: two workgroups, 512 + 488 picks (csr_count_half_body)
+                                   (3, 77, 13, 31, 128, 64)],     # 403 picks: two workgroups, 256 + 147 picks
+                         ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("dtype,type_id", [(torch.bfloat16, _abi.BF16), (torch.float32, _abi.F32)], ids=["bfloat16", "float32"])
-def test_table_is_the_stable_sort_of_the_picks_by_token(dtype, type_id):
-    B, T, E, K, I, J = 5, 50, 9, 11, 64, 32
+def test_table_is_the_stable_sort_of_the_picks_by_token(dtype, type_id, shape):
+    B, T, E, K, I, J = shape
     case = make_case(3, B, T, E, K, I, J, dtype)
     Ind = case["Ind"].clone()
     Ind[1, 2, 3] = T; Ind[2, 0, 0] = -5         # rejected picks have no place in any token's list
+    Ind[0, E - 1, K - 1] = -1; Ind[0, E // 2, :] = 7       # ... in either half; a token that a whole expert picks K times
     X, Wg, IndD = case["X"].to(DEV), case["Wg"].to(DEV), Ind.to(DEV)
     d = _abi.Dims(B, T, E, K, I, J)
     nb = _abi.lib().egs_routing_table_bytes(d, type_id)
