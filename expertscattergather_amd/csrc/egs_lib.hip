@@ -837,6 +837,9 @@ int scatter_fused(const void *Y, const void *W, const void *Ind, void *Out, cons
     p.perm_at = (int32_t)((int64_t)fp.experts_per_pass * d->K * kFusedCols * 4);
     p.cnt_at = p.perm_at + (int32_t)(NP * 4);
     p.zero_at = (int32_t)scatter_fused_zero_at(d->T, (int)NP, fp.experts_per_pass * d->K);
+    // where the rows come from a small-expert gather (256 picks of one expert per workgroup, row tiles mapped to XCDs), the
+    // batch elements of one of its row tiles - 256 / K of them - were written on one XCD
+    p.xcd_batch = (d->K == 32 || d->K == 64 || d->K == 128 || d->K == 256) ? 256 / d->K : 2;
     const bool nmajor = (w_layout == EGS_W_EJI);        // [E,J,I] = [E,R,N]
     if (act_dtype == EGS_F32)
         return nmajor ? launch_scatter_fused_ks<ElemF32, true>(p, R, lds, (int)blocks, nullptr, nullptr, s)

@@ -46,6 +46,7 @@ struct ScatterFusedParams {
     int32_t slices;         // N / kFusedCols
     int32_t perm_at, cnt_at;    // byte offsets of the table and of the sort's counters in dynamic LDS (rows start at 0)
     int32_t zero_at;            // ... and of 128 bytes of zeros (128-byte aligned), scatter_fused_zero_at()
+    int32_t xcd_batch;          // consecutive batch elements per XCD: 1, 2, 4 or 8
     int32_t experts_per_pass;   // MULTI: experts whose product rows are in LDS at a time (E otherwise)
     // TABLE: routing table built beforehand (seg [B][T+1], perm [B][E*K]); the workgroup copies its batch element's part
     // into LDS instead of sorting the picks itself
@@ -90,8 +91,11 @@ __device__ __forceinline__ void scatter_fused_body(const ScatterFusedParams &p, 
     // rows are fetched from memory once
     const int grp = block & 7, idx = block >> 3;
     const int qb = idx / p.slices, slice = idx % p.slices;
-    // XCD grp takes the batch elements 2 grp, 2 grp + 1 of every 16 (a last incomplete block: grp of every 8)
-    const int b = (qb | 1) < ((p.B + 7) >> 3) ? (qb >> 1) * 16 + grp * 2 + (qb & 1) : qb * 8 + grp;
+    // XCD grp takes runs of xcd_batch consecutive batch elements (a power of two up to 8: the batch elements of one 256-pick
+    // row tile of the gather that wrote this scatter's rows, which ran on the XCD of the same number), i.e. the elements
+    // xcd_batch * grp .. + xcd_batch - 1 of every 8 * xcd_batch; a last incomplete block: grp of every 8
+    const int nb = p.xcd_batch;
+    const int b = (qb | (nb - 1)) < ((p.B + 7) >> 3) ? ((qb / nb) * 8 + grp) * nb + (qb & (nb - 1)) : qb * 8 + grp;
     if (b >= p.B) return;
     const int c0 = slice * kFusedCols;
     const int T = p.T, E = p.E, K = p.K, N = p.N, NP = E * K;
