@@ -6,7 +6,11 @@
 // slab of gathered Xs rows (256 columns) and of Ys rows (BQ columns) is fetched with direct
 // 16-byte loads whose per-row byte offsets come from a small table decoded from Ind two slabs
 // ahead, and the MFMA fragments are produced by LDS transpose reads.  256 x BQ output tile,
-// 8 wavefronts (2 x 4), two slabs in flight, one barrier per slab.  Rows that do not exist
+// 8 wavefronts (2 x 4), one barrier per slab.  With 256 columns two 64 KB stages: one slab in
+// flight under the multiplication of another.  With 128 columns three 48 KB stages and two slabs
+// in flight; the offsets of 1024 reduction rows at a time are decoded before their first slab is
+// requested, so that no index load sits between the direct loads and the wait for a slab can
+// leave exactly the next slab's loads outstanding.  Rows that do not exist
 // (rejected picks, the ragged end of a split) get an offset outside the buffer descriptor and
 // arrive as zeros.
 //
@@ -23,26 +27,29 @@
 namespace egs {
 
 constexpr int kDlThreads = 512;      // 8 wavefronts
+constexpr int kDwChunkRows = 1024;   // three-stage form: reduction rows whose offsets are staged in LDS at a time
 
 struct DwDlParams {
     DwParams d;               // i_tiles / j_tiles count 256-row and BQ-column tiles here
     uint32_t x_bytes, y_bytes;
 };
 
-template <class TT, int BQ>
+template <class TT, int BQ, int NST = 2>
 __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
 {
     static_assert(TT::ES == 2, "16-bit element types");
     static_assert(BQ == 256 || BQ == 128, "column tile");
+    static_assert(NST == 2 || (NST == 3 && BQ == 128), "three stages of 48 KB fit, three of 64 KB do not");
     constexpr int BP = 256, BK = 64;
     constexpr int TP = 8, TQ = BQ / 64;                  // 16 x 16 tiles per wavefront: 128 x BQ/4
     constexpr int P_BYTES = BK * BP * 2, Q_BYTES = BK * BQ * 2, STAGE = P_BYTES + Q_BYTES;
     constexpr int QL = BQ / 64;                          // Q loads per wavefront per slab (P: 4)
     constexpr int QCR = BQ / 8;                          // 16-byte chunks per Q row
 
-    __shared__ __attribute__((aligned(1024))) char smem[2 * STAGE];
-    __shared__ uint32_t x_voff[2][BK];
-    __shared__ uint32_t y_voff[2][BK];
+    constexpr int TAB = NST == 2 ? 2 * BK : kDwChunkRows;  // two slabs' offsets, or a whole chunk's
+    __shared__ __attribute__((aligned(1024))) char smem[NST * STAGE];
+    __shared__ uint32_t x_voff[TAB];
+    __shared__ uint32_t y_voff[TAB];
 
     const DwParams &p = pp.d;
     int e, tile;
@@ -74,8 +81,8 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
     auto table_store = [&](int buf, bool ok, int64_t pick, int b, int32_t t) {
         if (tid < BK) {
             const bool live = ok && t >= 0;
-            x_voff[buf][tid] = live ? (uint32_t)(((int64_t)b * p.ldx_b + (int64_t)t * p.ldx_t) * 2) : kVoffInvalid;
-            y_voff[buf][tid] = live ? (uint32_t)(pick * p.J * 2) : kVoffInvalid;
+            x_voff[buf * BK + tid] = live ? (uint32_t)(((int64_t)b * p.ldx_b + (int64_t)t * p.ldx_t) * 2) : kVoffInvalid;
+            y_voff[buf * BK + tid] = live ? (uint32_t)(pick * p.J * 2) : kVoffInvalid;
         }
     };
 
@@ -98,17 +105,18 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
         q_row[jj] = row;
         q_col[jj] = j0 + lchunk * 8 < p.J ? (j0 + lchunk * 8) * 2 : -1;
     }
-    auto issue = [&](int buf, int stage) {
+    // tab0: where the slab's 64 rows start in the offset tables
+    auto issue = [&](int tab0, int stage) {
         char *base = smem + stage * STAGE;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-            uint32_t ro = x_voff[buf][p_row[jj]];
+            uint32_t ro = x_voff[tab0 + p_row[jj]];
             uint32_t vo = (ro == kVoffInvalid || p_col[jj] < 0) ? kVoffInvalid : ro + (uint32_t)p_col[jj];
             direct_load16(rs_x, vo, 0, base + (wave * 4 + jj) * 1024);
         }
 #pragma unroll
         for (int jj = 0; jj < QL; ++jj) {
-            uint32_t ro = y_voff[buf][q_row[jj]];
+            uint32_t ro = y_voff[tab0 + q_row[jj]];
             uint32_t vo = (ro == kVoffInvalid || q_col[jj] < 0) ? kVoffInvalid : ro + (uint32_t)q_col[jj];
             direct_load16(rs_y, vo, 0, base + P_BYTES + (wave * QL + jj) * 1024);
         }
@@ -134,32 +142,8 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
 #pragma unroll
         for (int y = 0; y < TQ; ++y) acc[x][y] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // ---------------- prologue: tables of slabs 0 and 1, loads of slab 0, index of slab 2 in flight
-    {
-        int64_t pick = 0; int b = 0;
-        bool ok = pick_of(0, pick, b);
-        int32_t t = ok ? load_token(p.Ind, p.ind_dtype, pick, p.T) : -1;
-        table_store(0, ok, pick, b, t);
-        ok = nslab > 1 && pick_of(1, pick, b);
-        t = ok ? load_token(p.Ind, p.ind_dtype, pick, p.T) : -1;
-        table_store(1, ok, pick, b, t);
-    }
-    __syncthreads();
-    if (nslab > 0) issue(0, 0);
-    int64_t nx_pick = 0; int nx_b = 0; int32_t nx_t = -1;
-    bool nx_ok = nslab > 2 && pick_of(2, nx_pick, nx_b);
-    if (nx_ok) nx_t = load_token(p.Ind, p.ind_dtype, nx_pick, p.T);
-
-    for (int sl = 0; sl < nslab; ++sl) {
-        wait_vmem<0>();
-        __syncthreads();            // slab sl landed; table of slab sl+1 visible; stage and table of slab sl-1 free
-        if (sl + 1 < nslab) issue((sl + 1) & 1, (sl + 1) & 1);
-        if (sl + 2 < nslab) table_store(sl & 1, nx_ok, nx_pick, nx_b, nx_t);     // read again after the next barrier
-        nx_ok = sl + 3 < nslab && pick_of(sl + 3, nx_pick, nx_b);
-        nx_t = -1;
-        if (nx_ok) nx_t = load_token(p.Ind, p.ind_dtype, nx_pick, p.T);
-
-        const char *tile_p = smem + (sl & 1) * STAGE;
+    auto multiply = [&](int stage) {
+        const char *tile_p = smem + stage * STAGE;
         const char *tile_q = tile_p + P_BYTES;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
@@ -181,6 +165,70 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
 #pragma unroll
                 for (int y = 0; y < TQ; ++y) mma_chunk<TT>(acc[x][y], qf[y], pf[x]);
         }
+    };
+
+    if constexpr (NST == 2) {
+    // ---------------- prologue: tables of slabs 0 and 1, loads of slab 0, index of slab 2 in flight
+    {
+        int64_t pick = 0; int b = 0;
+        bool ok = pick_of(0, pick, b);
+        int32_t t = ok ? load_token(p.Ind, p.ind_dtype, pick, p.T) : -1;
+        table_store(0, ok, pick, b, t);
+        ok = nslab > 1 && pick_of(1, pick, b);
+        t = ok ? load_token(p.Ind, p.ind_dtype, pick, p.T) : -1;
+        table_store(1, ok, pick, b, t);
+    }
+    __syncthreads();
+    if (nslab > 0) issue(0, 0);
+    int64_t nx_pick = 0; int nx_b = 0; int32_t nx_t = -1;
+    bool nx_ok = nslab > 2 && pick_of(2, nx_pick, nx_b);
+    if (nx_ok) nx_t = load_token(p.Ind, p.ind_dtype, nx_pick, p.T);
+
+    for (int sl = 0; sl < nslab; ++sl) {
+        wait_vmem<0>();
+        __syncthreads();            // slab sl landed; table of slab sl+1 visible; stage and table of slab sl-1 free
+        if (sl + 1 < nslab) issue(((sl + 1) & 1) * BK, (sl + 1) & 1);
+        if (sl + 2 < nslab) table_store(sl & 1, nx_ok, nx_pick, nx_b, nx_t);     // read again after the next barrier
+        nx_ok = sl + 3 < nslab && pick_of(sl + 3, nx_pick, nx_b);
+        nx_t = -1;
+        if (nx_ok) nx_t = load_token(p.Ind, p.ind_dtype, nx_pick, p.T);
+        multiply(sl & 1);
+    }
+    } else {
+    // ---------------- three stages, two slabs in flight.  The row offsets of a whole chunk of reduction rows are
+    // decoded from Ind before the chunk's first slab is requested, so that no index load sits between the
+    // direct loads of the pipeline: the wait for slab sl leaves exactly the loads of slab sl + 1 outstanding.
+    int stage = 0;
+    for (int chunk0 = row_begin; chunk0 < row_end; chunk0 += kDwChunkRows) {
+        const int chunk_rows = min(kDwChunkRows, row_end - chunk0);
+        const int nsl = (chunk_rows + BK - 1) / BK;
+        __syncthreads();            // the previous chunk's offsets and stages are no longer being read
+        for (int r = tid; r < nsl * BK; r += kDlThreads) {
+            const int m = chunk0 + r;
+            uint32_t xo = kVoffInvalid, yo = kVoffInvalid;
+            if (r < chunk_rows) {
+                const int b = m / p.K;
+                const int64_t pick = ((int64_t)b * p.E + e) * p.K + (m - b * p.K);
+                const int32_t t = load_token(p.Ind, p.ind_dtype, pick, p.T);
+                if (t >= 0) {
+                    xo = (uint32_t)(((int64_t)b * p.ldx_b + (int64_t)t * p.ldx_t) * 2);
+                    yo = (uint32_t)(pick * p.J * 2);
+                }
+            }
+            x_voff[r] = xo;
+            y_voff[r] = yo;
+        }
+        __syncthreads();
+        issue(0, stage);
+        if (nsl > 1) issue(BK, stage + 1 < NST ? stage + 1 : 0);
+        for (int sl = 0; sl < nsl; ++sl) {
+            if (sl + 1 < nsl) wait_vmem<4 + QL>(); else wait_vmem<0>();
+            __syncthreads();        // slab sl landed everywhere; the stage of slab sl - 1 is free
+            if (sl + 2 < nsl) issue((sl + 2) * BK, stage + 2 < NST ? stage + 2 : stage + 2 - NST);
+            multiply(stage);
+            if (++stage == NST) stage = 0;
+        }
+    }
     }
 
     // ---------------- epilogue: lane holds row i = i0 + wave_p0 + 16 x + a, columns j0 + wave_q0 + 16 y + 4 g .. + 3

@@ -1067,3 +1067,25 @@ def test_fp32_atomic_mode_at_zipf_sizes():
     finally:
         hk.set_scatter_mode("deterministic")
     assert_close(out, O.scatter_forward(np64(Y), np64(Ws), Ind.numpy(), T), torch.float32, "fp32 atomic, Zipf sizes")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
+@pytest.mark.parametrize("shape", [(3, 450, 256, 400, 136, 72),      # one split of 1200 rows per expert: a chunk of 1024 and a ragged one
+                                   (5, 500, 128, 450, 264, 128)],    # two splits of 1152 rows, two 256-row tiles of I, the second nearly empty
+                         ids=lambda s: "x".join(map(str, s)))
+def test_large_weight_gradient_with_128_columns_over_several_row_chunks(shape, dtype):
+    """The weight gradient of large shapes with at most 128 columns stages the row offsets of 1024 reduction rows at a
+    time and keeps two slabs in flight (reference kernel: egs/triton_kernels.py:261-356); more rows than one chunk,
+    a ragged last chunk and both layouts, against the oracle."""
+    B, T, E, K, I, J = shape
+    case = make_case(4242 + sum(shape), *shape, dtype)
+    X, Wg, Ws, Y, dOut, Ind = (dev(case[k]) for k in ("X", "Wg", "Ws", "Y", "dOut", "Ind"))
+    _, dWg = hk.expert_gather_backward_call(X, Wg, Ind, Y, torch.float32)
+    _, dWs = hk.expert_scatter_backward_call(Y, Ws, Ind, dOut, torch.float32)
+    torch.cuda.synchronize()
+    Indn = case["Ind"].to(torch.int64).numpy()
+    ref_g = O.gather_backward(np64(case["X"]), np64(case["Wg"]), Indn, np64(case["Y"]))[1]
+    ref_s = O.scatter_backward(np64(case["Y"]), np64(case["Ws"]), Indn, np64(case["dOut"]))[1]
+    assert_close(dWg, ref_g, dtype, f"dWg {shape} {dtype}")
+    assert_close(dWs, ref_s, dtype, f"dWs {shape} {dtype}")
