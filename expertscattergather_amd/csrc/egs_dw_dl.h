@@ -2,15 +2,16 @@
 //
 //   dW(e, i, j) = sum_{m in split s} Xs[b, Ind[m], i] * Ys[m, j]
 //
-// Both operands are [reduction][column] in memory, and they stay that way in LDS: each 64-row
+// Both operands are [reduction][column] in memory, and they stay that way in LDS: each BK-row
 // slab of gathered Xs rows (256 columns) and of Ys rows (BQ columns) is fetched with direct
-// 16-byte loads whose per-row byte offsets come from a small table decoded from Ind two slabs
-// ahead, and the MFMA fragments are produced by LDS transpose reads.  256 x BQ output tile,
-// 8 wavefronts (2 x 4), one barrier per slab.  With 256 columns two 64 KB stages: one slab in
-// flight under the multiplication of another.  With 128 columns three 48 KB stages and two slabs
-// in flight; the offsets of 1024 reduction rows at a time are decoded before their first slab is
-// requested, so that no index load sits between the direct loads and the wait for a slab can
-// leave exactly the next slab's loads outstanding.  Rows that do not exist
+// 16-byte loads whose per-row byte offsets come from a table decoded from Ind, and the MFMA
+// fragments are produced by LDS transpose reads.  256 x BQ output tile, 8 wavefronts (2 x 4),
+// one barrier per slab.  Stages: NST = 2 (64-row slabs) keeps one slab in flight under the
+// multiplication of another and decodes the offsets two slabs ahead inside the loop.  NST = 3
+// (128 columns, 48 KB stages of 64 rows) and NST = 4 (256 columns, 32 KB stages of 32 rows)
+// keep NST - 1 slabs in flight; the offsets of 1024 reduction rows at a time are decoded before
+// their first slab is requested, so that no index load sits between the direct loads and the
+// wait for a slab can leave exactly the later slabs' loads outstanding.  Rows that do not exist
 // (rejected picks, the ragged end of a split) get an offset outside the buffer descriptor and
 // arrive as zeros.
 //
@@ -34,17 +35,21 @@ struct DwDlParams {
     uint32_t x_bytes, y_bytes;
 };
 
-template <class TT, int BQ, int NST = 2>
+template <class TT, int BQ, int NST = 2, int BK = 64>
 __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
 {
     static_assert(TT::ES == 2, "16-bit element types");
     static_assert(BQ == 256 || BQ == 128, "column tile");
-    static_assert(NST == 2 || (NST == 3 && BQ == 128), "three stages of 48 KB fit, three of 64 KB do not");
-    constexpr int BP = 256, BK = 64;
+    static_assert(BK == 64 || BK == 32, "slab depth");
+    static_assert(NST >= 2 && NST <= 4 && (NST > 2 || BK == 64), "stages");
+    constexpr int BP = 256;
+    constexpr int KS = BK / 32;                          // matrix-instruction steps per slab
     constexpr int TP = 8, TQ = BQ / 64;                  // 16 x 16 tiles per wavefront: 128 x BQ/4
     constexpr int P_BYTES = BK * BP * 2, Q_BYTES = BK * BQ * 2, STAGE = P_BYTES + Q_BYTES;
-    constexpr int QL = BQ / 64;                          // Q loads per wavefront per slab (P: 4)
+    constexpr int PL = BK / 16;                          // P loads per wavefront per slab (1 KB = two rows each)
+    constexpr int QL = BK * BQ / 4096;                   // Q loads per wavefront per slab
     constexpr int QCR = BQ / 8;                          // 16-byte chunks per Q row
+    static_assert(NST * STAGE + (NST > 2 ? 8 * kDwChunkRows : 0) <= 160 * 1024, "LDS of a CU");
 
     constexpr int TAB = NST == 2 ? 2 * BK : kDwChunkRows;  // two slabs' offsets, or a whole chunk's
     __shared__ __attribute__((aligned(1024))) char smem[NST * STAGE];
@@ -88,10 +93,10 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
 
     // ---------------- loaders.  P tile [64][256]: load j covers rows 2j, 2j+1 (lane l: row 2j + l/32,
     // physical chunk l%32).  Q tile [64][BQ]: 64/QCR rows per load.
-    int p_row[4], p_col[4], q_row[QL], q_col[QL];      // tile row a load lands on, byte offset of its column chunk (-1: outside)
+    int p_row[PL], p_col[PL], q_row[QL], q_col[QL];    // tile row a load lands on, byte offset of its column chunk (-1: outside)
 #pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-        int row = (wave * 4 + jj) * 2 + (lane >> 5);
+    for (int jj = 0; jj < PL; ++jj) {
+        int row = (wave * PL + jj) * 2 + (lane >> 5);
         int pc = lane & 31;
         int lchunk = ((((pc >> 1) ^ tr_swizzle(row)) << 1) | (pc & 1));
         p_row[jj] = row;
@@ -109,10 +114,10 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
     auto issue = [&](int tab0, int stage) {
         char *base = smem + stage * STAGE;
 #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
+        for (int jj = 0; jj < PL; ++jj) {
             uint32_t ro = x_voff[tab0 + p_row[jj]];
             uint32_t vo = (ro == kVoffInvalid || p_col[jj] < 0) ? kVoffInvalid : ro + (uint32_t)p_col[jj];
-            direct_load16(rs_x, vo, 0, base + (wave * 4 + jj) * 1024);
+            direct_load16(rs_x, vo, 0, base + (wave * PL + jj) * 1024);
         }
 #pragma unroll
         for (int jj = 0; jj < QL; ++jj) {
@@ -126,9 +131,9 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
     // 16 t + 4 (a%4) of tile t, and receives column 16 t + a of rows 8 g + 4 h .. + 3
     const int a = lane & 15, g = lane >> 4;
     const int wave_p0 = (wave >> 2) * 128, wave_q0 = (wave & 3) * (BQ / 4);
-    int p_at[2][2], q_at[2][2];
+    int p_at[KS][2], q_at[KS][2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
+    for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             int row = ks * 32 + g * 8 + h * 4 + (a >> 2);
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
         const char *tile_p = smem + stage * STAGE;
         const char *tile_q = tile_p + P_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < KS; ++ks) {
             u32x4 pf[TP], qf[TQ];
 #pragma unroll
             for (int x = 0; x < TP; ++x) {
@@ -168,6 +173,7 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
     };
 
     if constexpr (NST == 2) {
+    static_assert(NST > 2 || (PL == 4 && BK == 64), "the two-stage form is written for 64-row slabs");
     // ---------------- prologue: tables of slabs 0 and 1, loads of slab 0, index of slab 2 in flight
     {
         int64_t pick = 0; int b = 0;
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
         multiply(sl & 1);
     }
     } else {
-    // ---------------- three stages, two slabs in flight.  The row offsets of a whole chunk of reduction rows are
+    // ---------------- three or four stages, all but one in flight.  The row offsets of a whole chunk of reduction rows are
     // decoded from Ind before the chunk's first slab is requested, so that no index load sits between the
     // direct loads of the pipeline: the wait for slab sl leaves exactly the loads of slab sl + 1 outstanding.
     int stage = 0;
@@ -219,12 +225,17 @@ __global__ __launch_bounds__(kDlThreads) void dw_dl_kernel(DwDlParams pp)
             y_voff[r] = yo;
         }
         __syncthreads();
-        issue(0, stage);
-        if (nsl > 1) issue(BK, stage + 1 < NST ? stage + 1 : 0);
+#pragma unroll
+        for (int st = 0; st < NST - 1; ++st)
+            if (st < nsl) issue(st * BK, stage + st < NST ? stage + st : stage + st - NST);
         for (int sl = 0; sl < nsl; ++sl) {
-            if (sl + 1 < nsl) wait_vmem<4 + QL>(); else wait_vmem<0>();
+            // slab sl has landed once only the slabs requested after it (at most NST - 2) are outstanding
+            const int later = min(nsl - 1 - sl, NST - 2);
+            if (NST >= 4 && later >= 2) wait_vmem<(NST >= 4 ? 2 : 0) * (PL + QL)>();
+            else if (later >= 1) wait_vmem<PL + QL>();
+            else wait_vmem<0>();
             __syncthreads();        // slab sl landed everywhere; the stage of slab sl - 1 is free
-            if (sl + 2 < nsl) issue((sl + 2) * BK, stage + 2 < NST ? stage + 2 : stage + 2 - NST);
+            if (sl + NST - 1 < nsl) issue((sl + NST - 1) * BK, stage + NST - 1 < NST ? stage + NST - 1 : stage - 1);
             multiply(stage);
             if (++stage == NST) stage = 0;
         }

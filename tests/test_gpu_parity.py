@@ -1072,11 +1072,12 @@ def test_fp32_atomic_mode_at_zipf_sizes():
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bfloat16", "float16"])
 @pytest.mark.parametrize("shape", [(3, 450, 256, 400, 136, 72),      # one split of 1200 rows per expert: a chunk of 1024 and a ragged one
-                                   (5, 500, 128, 450, 264, 128)],    # two splits of 1152 rows, two 256-row tiles of I, the second nearly empty
+                                   (5, 500, 128, 450, 264, 128),     # two splits of 1152 rows, two 256-row tiles of I, the second nearly empty
+                                   (5, 600, 40, 420, 264, 200)],     # 256-column tiles in four stages of 32 rows: 2100 rows, one split
                          ids=lambda s: "x".join(map(str, s)))
-def test_large_weight_gradient_with_128_columns_over_several_row_chunks(shape, dtype):
-    """The weight gradient of large shapes with at most 128 columns stages the row offsets of 1024 reduction rows at a
-    time and keeps two slabs in flight (reference kernel: egs/triton_kernels.py:261-356); more rows than one chunk,
+def test_large_weight_gradient_over_several_row_chunks(shape, dtype):
+    """The weight gradient of large shapes stages the row offsets of 1024 reduction rows at a time and keeps two or
+    three slabs in flight (reference kernel: egs/triton_kernels.py:261-356); more rows than one chunk,
     a ragged last chunk and both layouts, against the oracle."""
     B, T, E, K, I, J = shape
     case = make_case(4242 + sum(shape), *shape, dtype)
