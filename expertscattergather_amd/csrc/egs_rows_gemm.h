@@ -35,7 +35,8 @@ struct RowsGemmParams {
     uint32_t a_bytes;       // extent of A in bytes when it is below 2 GiB, else 0 (direct-load kernel only)
     // routing table of the scatter built by the first csr_blocks (= B) workgroups of the product launch
     // (direct-load kernel only; csr_done reports that the launch took it along)
-    int32_t csr_blocks, csr_done, csr_threads;
+    // csr_parts workgroups share a batch element's table (csr_blocks = B * csr_parts; set by the launcher)
+    int32_t csr_blocks, csr_done, csr_threads, csr_parts;
     int32_t *seg_off, *perm, *rank_tmp, *long_tab;
 };
 

@@ -85,8 +85,9 @@ __global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGe
         // builds it here (csr_threads of the workgroup, histograms in the slab buffers) instead of in a launch of its own
         if (block < p.csr_blocks) {
             if (tid >= p.csr_threads) return;
-            csr_count_body(reinterpret_cast<int32_t *>(smem), block, block, tid, p.csr_threads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
-                           p.seg_off, p.perm, p.rank_tmp, p.long_tab);
+            const int cb = block / p.csr_parts;
+            csr_count_body(reinterpret_cast<int32_t *>(smem), cb, cb, tid, p.csr_threads, p.Ind, p.ind_dtype, p.T, p.E * p.K,
+                           p.seg_off, p.perm, p.rank_tmp, p.long_tab, NoPrefetch(), block - cb * p.csr_parts, p.csr_parts);
             return;
         }
         block -= p.csr_blocks;

@@ -43,6 +43,16 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                     p.csr_threads = 512;            // as many wavefronts as the histograms leave room for
                     while (p.csr_threads > kWave && csr_count_lds(p.T, p.csr_threads / kWave) > smem) p.csr_threads >>= 1;
                     if (GATHER || csr_count_lds(p.T, p.csr_threads / kWave) > smem) p.csr_blocks = 0;
+                    // many picks per batch element: several workgroups per table, each ranking a share whose wavefront
+                    // slices (512 picks) stay in registers; one workgroup ranking 32768 picks outlasts the product tiles
+                    // of its launch (C3: 100 against 38 us; with eight parts the launch takes 54 us, one more round of workgroups)
+                    p.csr_parts = 1;
+                    if (p.csr_blocks > 0) {
+                        const int64_t per = (int64_t)(p.csr_threads / kWave) * 512;
+                        const int64_t parts = ((int64_t)p.E * p.K + per - 1) / per;
+                        p.csr_parts = (int)(parts < 1 ? 1 : parts > 8 ? 8 : parts);
+                        p.csr_blocks *= p.csr_parts;
+                    }
                     grid += p.csr_blocks;
                     if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
                     p.csr_done = p.csr_blocks > 0;

@@ -146,13 +146,18 @@ static __global__ __launch_bounds__(kWave) void csr_build_kernel(const void *Ind
 // offsets are left in sh_cnt[NW * T ..]).  `after_token_loads` runs once the tokens have been decoded, before the
 // table is built: a caller's own prefetches belong there, they travel while the table is built and the wait
 // for the tokens does not have to cover them.
+// `parts` > 1: the batch element's table is built by `parts` workgroups, this one being number `part`.  It ranks only
+// its own contiguous share of the picks (so that a wavefront's slice stays in registers where one workgroup's would
+// not) and merely counts the others, with LDS atomics: the picks before its share into the first wavefront's
+// counters, which therefore start at that count and carry it into every rank and prefix, the picks after its share
+// into the token totals.  Every part computes the same offsets; part 0 stores them and lists the long tokens.
 struct NoPrefetch { __device__ __forceinline__ void operator()() const {} };
 
 template <class AfterTokenLoads = NoPrefetch>
 __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b, int tid, int nthreads, const void *Ind,
                                                int32_t ind_dtype, int32_t T, int32_t N, int32_t *seg_off,
                                                int32_t *perm, int32_t *rank_tmp, int32_t *long_tab,
-                                               AfterTokenLoads after_token_loads = AfterTokenLoads())
+                                               AfterTokenLoads after_token_loads = AfterTokenLoads(), int part = 0, int parts = 1)
 {
     constexpr int MAXC = 8;                             // 64-pick chunks whose tokens (and ranks) are held in registers at a time
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), NW = nthreads >> 6;
@@ -160,8 +165,10 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
     int32_t *tok_start = sh_cnt + (size_t)NW * T;       // [T + 1]
     const int64_t base_pick = (int64_t)b * N;           // where this batch element's picks start in Ind
     const int64_t out_pick = (int64_t)out_b * N;        // ... and in perm / rank_tmp
-    const int slice = ((N + NW - 1) / NW + 63) & ~63;
-    const int q_begin = wave * slice, q_end = min(N, q_begin + slice);
+    const int own = parts > 1 ? (((N + parts - 1) / parts + 63) & ~63) : N;
+    const int own_begin = min(N, part * own), own_end = min(N, own_begin + own);
+    const int slice = ((own_end - own_begin + NW - 1) / NW + 63) & ~63;
+    const int q_begin = own_begin + wave * slice, q_end = min(own_end, q_begin + slice);
     const bool in_regs = slice <= MAXC * kWave;
 
     // tokens of the slice go in flight before anything else.  Only the loads: decoding a token here would make
@@ -179,6 +186,26 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
     // accesses happen in order, so no barrier is needed before it ranks
     for (int i = lane; i < T; i += kWave) cnt_store(&hist[i], 0);
     __builtin_amdgcn_wave_barrier();
+    if (parts > 1) {
+        for (int i = tid; i <= T; i += nthreads) cnt_store(&tok_start[i], 0);
+        __syncthreads();                                // every counter is clear
+        constexpr int U = 16;                           // token loads in flight per thread
+        for (int q0 = 0; q0 < N; q0 += U * nthreads) {
+            int32_t ft[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = q0 + u * nthreads + tid;
+                const bool foreign = q < N && (q < own_begin || q >= own_end);
+                ft[u] = foreign ? load_token(Ind, ind_dtype, base_pick + q, T) : -1;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int q = q0 + u * nthreads + tid;
+                if (ft[u] >= 0) atomicAdd(q < own_begin ? &sh_cnt[ft[u]] : &tok_start[ft[u]], 1);
+            }
+        }
+        __syncthreads();                                // the first wavefront's counters start at the picks before this share
+    }
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
         const int q = q_begin + c * kWave + lane;
@@ -253,7 +280,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
             if (w < NW) sh_cnt[(size_t)w * T + t] = run;
             run += c[w];
         }
-        tok_start[t] = run;
+        tok_start[t] = parts > 1 ? run + tok_start[t] : run;     // + the picks after this share
     }
     __syncthreads();
     {   // exclusive scan of the totals over tokens: each wavefront scans a contiguous part,
@@ -282,7 +309,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
         if (tid == 0) tok_start[T] = total;
     }
     __syncthreads();
-    if (seg_off != nullptr)
+    if (seg_off != nullptr && part == 0)
         for (int t = tid; t <= T; t += nthreads) seg_off[(size_t)out_b * (T + 1) + t] = tok_start[t];
     if (in_regs) {
 #pragma unroll
@@ -303,7 +330,7 @@ __device__ __forceinline__ void csr_count_body(int32_t *sh_cnt, int b, int out_b
                 if (tk[c] >= 0) perm[out_pick + tok_start[tk[c]] + hist[tk[c]] + rr[c]] = q0 + c * kWave + lane;
         }
     }
-    emit_long_tokens(tok_start, T, N, long_tab, out_b, tid, nthreads);
+    if (part == 0) emit_long_tokens(tok_start, T, N, long_tab, out_b, tid, nthreads);
 }
 
 // The same table built by TWO workgroups per batch element (`h` = 0 or 1), for the case where it rides in a launch that has
