@@ -53,7 +53,8 @@ __device__ __forceinline__ int tr_swizzle(int row) { return (row & 3) | (((row >
 template <int CR> __device__ __forceinline__ int kmajor_key_rows(int row) { return CR == 8 ? (row & 7) : ((row >> 2) & 3); }
 
 template <class TT, int WES, int BM, int BN, int BK, int NSTAGE, bool GATHER, bool W_TRANS, int EPI>
-__global__ __launch_bounds__(dl_threads(BM, BN)) void rows_gemm_dl_kernel(RowsGemmParams p)
+// (four-wavefront workgroups on 32-deep slabs are meant to run two to a CU: at most 256 registers per wavefront)
+__global__ __launch_bounds__(dl_threads(BM, BN), (BK == 32 && dl_threads(BM, BN) == 256) ? 2 : 1) void rows_gemm_dl_kernel(RowsGemmParams p)
 {
     static_assert(TT::ES == 2, "16-bit element types");
     static_assert(EPI == EPI_STORE || EPI == EPI_STORE_F32, "plain stores only");

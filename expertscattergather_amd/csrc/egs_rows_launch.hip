@@ -66,8 +66,11 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
         }
     } else {
         // 65..191 output columns.  The gathers of large, well-formed 16-bit shapes take the direct-to-LDS
-        // pipeline with 256 x 128 x 64 tiles (four wavefronts, two stages; 32-deep slabs with three workgroups per
-        // CU and a third stage measured the same or slower)
+        // pipeline with 256 x 128 tiles of four wavefronts in three stages of 32-deep slabs (75 KB), compiled for two
+        // wavefronts per SIMD so that TWO workgroups share a CU and one's loads and stores run under the other's
+        // matrix instructions: C4 gather 29.5 -> 21.5 us against 64-deep slabs in two stages with one workgroup per
+        // CU.  (Left to itself the compiler gives a four-wavefront workgroup 144 + 128 accumulator registers, which
+        // keeps a second workgroup off the CU whatever the LDS size.)
         if constexpr (TT::ES == 2 && WES == 2 && GATHER && EPI == EPI_STORE) {
             const bool dl = !g_force_generic && Me >= 256 && p.R >= 128 && p.R % 64 == 0 && p.N % 8 == 0 && p.a_vec && p.w_vec &&
                             p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && p.w_scale == nullptr && aligned_to(p.C, 16);
@@ -76,7 +79,7 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                 int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
                 if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
                 p.csr_blocks = 0;
-                hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, 2, 256, 128, 64, 2, true, W_TRANS, EPI_STORE>), dim3((unsigned)grid),
+                hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, 2, 256, 128, 32, 3, true, W_TRANS, EPI_STORE>), dim3((unsigned)grid),
                                    dim3(dl_threads(256, 128)), 0, s, p);
                 EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
                 return EGS_OK;
