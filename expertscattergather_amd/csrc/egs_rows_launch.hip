@@ -31,8 +31,10 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
             p.m_tiles = ceil_div(Me, BM); p.n_tiles = ceil_div(p.N, BN);
             int64_t grid = (int64_t)8 * e_groups * p.m_tiles * p.n_tiles;
             if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
-            // well-formed shapes take the direct-to-LDS pipeline (256 x 256 x 64 slabs, two stages; a 128 x 256 x 32
-            // shape with two or three workgroups per CU was measured slower at every benchmark configuration)
+            // well-formed shapes take the direct-to-LDS pipeline (256 x 256 x 64 slabs, two stages).  256 x 128 tiles of
+            // four wavefronts on 32-deep slabs, two workgroups to a CU, measured for these shapes: gather at C3 156 -> 170 us
+            // (gathered rows fetched once per column tile), fp32 product rows at C3 38.7 -> 40.2 us per group and at C5
+            // 1.80 -> 2.09 ms; at C4 31.9 -> 28.7 us, which the table workgroups riding along take back
             const bool dl = !g_force_generic && p.R % 64 == 0 && p.N % (WES == 1 ? 16 : 8) == 0 && p.a_vec && p.w_vec &&
                             p.a_bytes != 0 && (uint64_t)p.R * p.N * 2 < (1ull << 31) && (WES == 1 || p.w_scale == nullptr) &&
                             (WES == 2 || aligned_to(p.W, 16)) &&
