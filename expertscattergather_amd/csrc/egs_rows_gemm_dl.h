@@ -31,11 +31,12 @@
 
 namespace egs {
 
-// LDS bytes of one workgroup: slab stages, then the row tables (4 + 8 bytes per tile row)
-__host__ __device__ constexpr int dl_stage_bytes(int BM, int BN, int BK) { return (BM + BN) * BK * 2; }
-__host__ __device__ constexpr int dl_smem_bytes(int BM, int BN, int BK, int NSTAGE)
+// LDS bytes of one workgroup: slab stages (rows in 16-bit elements, weights in WES-byte elements), then the row tables
+// (4 + 8 bytes per tile row)
+__host__ __device__ constexpr int dl_stage_bytes(int BM, int BN, int BK, int WES = 2) { return (BM * 2 + BN * WES) * BK; }
+__host__ __device__ constexpr int dl_smem_bytes(int BM, int BN, int BK, int NSTAGE, int WES = 2)
 {
-    return NSTAGE * dl_stage_bytes(BM, BN, BK) + BM * 12;
+    return NSTAGE * dl_stage_bytes(BM, BN, BK, WES) + BM * 12;
 }
 // the scatter variants of the one-workgroup-per-CU shape reserve more, so that the routing-table
 // workgroups riding along have room for eight wavefronts' histograms at T = 4096
@@ -68,13 +69,13 @@ __global__ __launch_bounds__(dl_threads(BM, BN), (BK == 32 && dl_threads(BM, BN)
     constexpr int TM = 8, TN = 4;                        // 16 x 16 tiles per wavefront: 128 x 64
     constexpr int KSTEPS = BK / 32;
     constexpr int CR = BK / 8;                           // 16-byte chunks per K-major row
-    constexpr int P_BYTES = BM * BK * 2, STAGE = dl_stage_bytes(BM, BN, BK);
+    constexpr int P_BYTES = BM * BK * 2, STAGE = dl_stage_bytes(BM, BN, BK, WES);
     constexpr int PL = BM * CR / 64 / NW;                // loads per wavefront and slab: row side,
     constexpr int WROW = BN * 2;                         // bytes of a [reduction][column] tile row (16-bit)
     constexpr int QL = W_FP8 ? BK / 4 / NW : (W_TRANS ? BK * WROW / 1024 / NW : BN * CR / 64 / NW);   // weight side
     static_assert(PL >= 1 && QL >= 1 && PL + QL < 16, "loads per slab");
 
-    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? dl_smem_bytes(BM, BN, BK, NSTAGE)
+    __shared__ __attribute__((aligned(1024))) char smem[GATHER ? dl_smem_bytes(BM, BN, BK, NSTAGE, WES)
                                                                : dl_smem_bytes_scatter(BM, BN, BK, NSTAGE)];
     uint32_t *a_voff = reinterpret_cast<uint32_t *>(smem + NSTAGE * STAGE);
     int64_t *c_off = reinterpret_cast<int64_t *>(smem + NSTAGE * STAGE + BM * 4);

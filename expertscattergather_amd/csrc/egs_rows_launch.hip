@@ -58,6 +58,12 @@ int launch_rows_gemm_cfg(RowsGemmParams &p, hipStream_t s)
                     grid += p.csr_blocks;
                     if (grid > INT32_MAX) return EGS_ERR_BAD_SHAPE;
                     p.csr_done = p.csr_blocks > 0;
+                    if constexpr (WES == 1 && GATHER) {
+                        // fp8 weights: a stage is 32 KB of rows + 16 KB of weight bytes, so three fit (C5 gather 1058 -> 1024 us)
+                        hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, 256, 256, 64, 3, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(512), 0, s, p);
+                        EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
+                        return EGS_OK;
+                    }
                     hipLaunchKernelGGL((rows_gemm_dl_kernel<TT, WES, 256, 256, 64, 2, GATHER, W_TRANS, EPI>), dim3((unsigned)grid), dim3(512), 0, s, p);
                     EGS_CHECK_LAUNCH("rows_gemm_dl_kernel");
                     return EGS_OK;
