@@ -1090,3 +1090,43 @@ def test_large_weight_gradient_over_several_row_chunks(shape, dtype):
     ref_s = O.scatter_backward(np64(case["Y"]), np64(case["Ws"]), Indn, np64(case["dOut"]))[1]
     assert_close(dWg, ref_g, dtype, f"dWg {shape} {dtype}")
     assert_close(dWs, ref_s, dtype, f"dWs {shape} {dtype}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["deterministic", "atomic"])
+@pytest.mark.parametrize("shape", [(2, 777, 37, 130, 256, 128),      # 4810 picks per batch element: two table workgroups, ragged shares
+                                   (3, 1500, 70, 129, 192, 128),     # 9030 picks: three
+                                   (2, 3000, 140, 150, 192, 128)],   # 21000 picks and 3000 tokens: six, and wavefront slices of 512
+                         ids=lambda s: "x".join(map(str, s)))
+def test_routing_table_built_by_several_workgroups(shape, mode):
+    """Batch elements with more than 4096 picks have their routing table built by several workgroups, each ranking a share
+    of the picks and counting the rest (the reference's scatter, egs/triton_kernels.py:156-247, has no table: it adds with
+    atomics).  Hot tokens, rejected picks and odd sizes, against the oracle, and the same bits on a second call."""
+    B, T, E, K, I, J = shape
+    dtype = torch.bfloat16
+    case = make_case(977 + sum(shape), *shape, dtype)
+    Ind = case["Ind"].clone()
+    g = torch.Generator().manual_seed(5)
+    hot = torch.rand(B, E, K, generator=g) < 0.2
+    Ind[hot] = 7                                           # a fifth of all picks on one token: segments cut into chunks
+    Ind[0, 0, 0] = T; Ind[-1, E // 2, 3] = -1; Ind[-1, E - 1, K - 1] = 10 ** 9
+    bad = (Ind < 0) | (Ind >= T)
+    Y, Ws = dev(case["Y"]), dev(case["Ws"])
+    from expertscattergather_amd import _abi
+    hk.set_scatter_mode(mode)
+    try:
+        with _abi.launch_log() as log:
+            out = hk.expert_scatter_forward_call(Y, Ws, dev(Ind), T, torch.float32)
+        again = hk.expert_scatter_forward_call(Y, Ws, dev(Ind), T, torch.float32)
+        torch.cuda.synchronize()
+    finally:
+        hk.set_scatter_mode("deterministic")
+    # the table rides in the product launch (no table kernel of its own), which is where it is built in parts
+    assert "rows_gemm_dl_kernel" in log.kernels and not any(k.startswith("csr_") for k in log.kernels), log.kernels
+    safe = Ind.clone(); safe[bad] = 0
+    mask = (~bad).numpy()[..., None]
+    ref = O.scatter_forward(np64(case["Y"]) * mask, np64(case["Ws"]), safe.numpy(), T)
+    # the hot token sums a few thousand products: its row sets the scale of the comparison
+    assert_close(out, ref, dtype, f"out {shape} {mode}")
+    if mode == "deterministic":
+        assert torch.equal(out, again)
