@@ -630,6 +630,12 @@ int launch_routing_table(const void *Ind, int ind_dtype, const egs_dims *d, int3
     return EGS_OK;
 }
 
+template <class TT, class PT>
+void launch_segment_sum8(const SegSumParams &sp, int seg_blocks, hipStream_t s)
+{
+    hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 8>), dim3(seg_blocks), dim3(kThreads), 0, s, sp);
+}
+
 // fixed-order reduction of the product rows per token; when `reduce` is given (and qualifies) the
 // second pass of that weight gradient shares the launch
 int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, const int32_t *perm, int32_t *long_tab,
@@ -637,7 +643,11 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
 {
     const int N = d->E * d->K;
     const bool vw4 = d->I % 4 == 0 && aligned_to(Out, 16);
-    const int iv = vw4 ? d->I / 4 : d->I;
+    // eight elements of a row per thread (16 bytes of a 16-bit row, two 16-byte loads of an fp32 row): half the threads,
+    // table look-ups and address arithmetic per row
+    const bool vw8 = vw4 && d->I % 8 == 0 && aligned_to(rows, 16) &&
+                     !(reduce != nullptr && reduce->done && reduce->q.S > 1);
+    const int iv = vw8 ? d->I / 8 : vw4 ? d->I / 4 : d->I;
     SegSumParams sp;
     memset(&sp, 0, sizeof(sp));
     sp.P = rows; sp.seg_off = seg_off; sp.perm = perm; sp.out = (char *)Out;
@@ -657,6 +667,7 @@ int launch_segment_sum(const void *rows, bool rows_f32, const int32_t *seg_off, 
         if (fuse) hipLaunchKernelGGL((segsum_dwreduce_kernel<TT, PT, 4>), dim3(seg_blocks + red_blocks), dim3(kThreads), 0, \
                                      s, sp, seg_blocks, (const float *)reduce->q.part, reduce->q.dW, reduce->q.S,           \
                                      reduce->w_elems / 4, reduce->q.out_dtype);                                             \
+        else if (vw8) launch_segment_sum8<TT, PT>(sp, seg_blocks, s);                                                       \
         else if (vw4) hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 4>), dim3(seg_blocks), dim3(kThreads), 0, s, sp);      \
         else hipLaunchKernelGGL((segment_sum_kernel<TT, PT, 1>), dim3(seg_blocks), dim3(kThreads), 0, s, sp);               \
     } while (0)

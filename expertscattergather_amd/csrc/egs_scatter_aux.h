@@ -545,6 +545,7 @@ struct SegSumParams {
 template <class TT, class PT, int VW>
 __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const int bx, const int by)
 {
+    static_assert(VW == 1 || VW == 4 || VW == 8, "a thread takes 1, 4 or 8 elements of a row");
     // 2^tpr_log2 threads share an output row (VW columns each, looping if the row is wider);
     // bx selects a group of rows of batch element by (+ a stride loop over b)
     const PT *P = reinterpret_cast<const PT *>(sp.P);
@@ -591,42 +592,50 @@ __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const i
         const int32_t *pb = perm + (size_t)b * N;
         const PT *Pb = P + (size_t)b * N * I + (size_t)iv * VW;
         int s = s0;
-        if constexpr (VW == 4) {
-            typedef typename std::conditional<sizeof(PT) == 4, f32x4, u32x2>::type vec_t;
+        if constexpr (VW >= 4) {
+            struct alignas(16) F32x8 { f32x4 lo, hi; };
+            typedef typename std::conditional<sizeof(PT) == 4, typename std::conditional<VW == 8, F32x8, f32x4>::type,
+                                              typename std::conditional<VW == 8, u32x4, u32x2>::type>::type vec_t;
             auto add_vec = [&](const vec_t &v) {
-                if constexpr (sizeof(PT) == 4) {
+                if constexpr (sizeof(PT) == 4 && VW == 8) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) { acc[x] += v.lo[x]; acc[4 + x] += v.hi[x]; }
+                } else if constexpr (sizeof(PT) == 4) {
 #pragma unroll
                     for (int x = 0; x < 4; ++x) acc[x] += v[x];
                 } else {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) {
+                    for (int x = 0; x < VW; ++x) {
                         uint32_t hbits = (v[x >> 1] >> (16 * (x & 1))) & 0xffffu;
                         acc[x] += TT::ID == 2 ? bf16_bits_to_f32(hbits) : f16_bits_to_f32(hbits);
                     }
                 }
             };
-            // long segments (hot tokens): 16 rows in flight per thread; added in table order all the same
-            for (; s + 16 <= s1; s += 16) {
-                int q[16];
-                vec_t v[16];
+            // long segments (hot tokens): 16 rows (256 bytes) in flight per thread; added in table order all the same
+            constexpr int LB = sizeof(vec_t) == 32 ? 8 : 16;
+            for (; s + LB <= s1; s += LB) {
+                int q[LB];
+                vec_t v[LB];
 #pragma unroll
-                for (int u = 0; u < 16; ++u) q[u] = pb[s + u];
+                for (int u = 0; u < LB; ++u) q[u] = pb[s + u];
 #pragma unroll
-                for (int u = 0; u < 16; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
+                for (int u = 0; u < LB; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
 #pragma unroll
-                for (int u = 0; u < 16; ++u) add_vec(v[u]);
+                for (int u = 0; u < LB; ++u) add_vec(v[u]);
             }
-            for (; s < s1; s += 4) {
-                const int n4 = min(4, s1 - s);
-                int q[4];
-                vec_t v[4];
+            // 16-bit rows are half the bytes per load: twice the rows per round trip keep as many bytes in flight
+            constexpr int RB = sizeof(PT) == 2 ? 8 : 4;
+            for (; s < s1; s += RB) {
+                const int nb = min(RB, s1 - s);
+                int q[RB];
+                vec_t v[RB];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) q[u] = pb[min(s + u, s1 - 1)];
+                for (int u = 0; u < RB; ++u) q[u] = pb[min(s + u, s1 - 1)];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
+                for (int u = 0; u < RB; ++u) v[u] = *reinterpret_cast<const vec_t *>(Pb + (size_t)q[u] * I);
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    if (u < n4) add_vec(v[u]);
+                for (int u = 0; u < RB; ++u)
+                    if (u < nb) add_vec(v[u]);
             }
         } else {
             for (; s < s1; ++s) add_row(Pb + (size_t)pb[s] * I);
@@ -634,11 +643,17 @@ __device__ __forceinline__ void segment_sum_body(const SegSumParams &sp, const i
         size_t at = row * I + (size_t)iv * VW;
         if constexpr (TT::ES == 4) {
             float *dst = reinterpret_cast<float *>(out) + at;
-            if constexpr (VW == 4) *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[0], acc[1], acc[2], acc[3]};
+            if constexpr (VW >= 4) *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[0], acc[1], acc[2], acc[3]};
             else dst[0] = acc[0];
+            if constexpr (VW == 8) *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[4], acc[5], acc[6], acc[7]};
         } else {
             uint16_t *dst = reinterpret_cast<uint16_t *>(out) + at;
-            if constexpr (VW == 4) {
+            if constexpr (VW == 8) {
+                u32x4 w;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) w[x] = pack2<TT>(acc[2 * x], acc[2 * x + 1]);
+                *reinterpret_cast<u32x4 *>(dst) = w;
+            } else if constexpr (VW == 4) {
                 u32x2 w;
                 w[0] = pack2<TT>(acc[0], acc[1]);
                 w[1] = pack2<TT>(acc[2], acc[3]);
@@ -801,7 +816,7 @@ __device__ __forceinline__ void segment_sum_dispatch(const SegSumParams &sp, con
     const int slots = long_max_slots(sp.N);
     const int long_blocks = sp.B * slots;
     if (block < long_blocks) {
-        segment_sum_long_body<TT, PT, VW>(sp, block / slots, block % slots);
+        segment_sum_long_body<TT, PT, (VW == 8 ? 4 : VW)>(sp, block / slots, block % slots);   // its partial rows are laid out for 4
     } else {
         const int sb = block - long_blocks;
         segment_sum_body<TT, PT, VW>(sp, sb % sp.gx, sb / sp.gx);
